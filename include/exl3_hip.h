@@ -1,0 +1,179 @@
+/*
+ * C ABI of the MI355X (gfx950) EXL3 quantized-linear library, libexl3_hip.so.
+ *
+ * Every entry point takes raw device pointers, sizes and a HIP stream
+ * (hipStream_t passed as void*, NULL = the default stream) and returns an int
+ * status: 0 on success, a negative EXL3_E_* code otherwise. Nothing throws
+ * across the boundary and nothing is allocated or freed by the library: the
+ * caller owns every buffer, including the workspace. All launches are
+ * asynchronous on the given stream. Argument checks happen on the host before
+ * any launch, mirroring the reference, whose kernels have no error channel and
+ * whose host wrappers raise ValueError first
+ * (ponyexl3/ref/layer.py:35-44, ponyexl3/mlx/gemv_metal.py:1354-1372).
+ *
+ * Tensor contract (ponyexl3/ref/layer.py:12-44):
+ *   trellis  uint16 [in_tiles][out_tiles][16*K], in_tiles = in/16, out_tiles = out/16
+ *   suh/svh  fp16 per-channel multipliers [in] / [out] (general scales, not only +-1)
+ *   K        bits per weight, 1..8
+ *   cb       codebook id: 0 = 3INST (default), 1 = MCG, 2 = MUL1
+ *            (ponyexl3/ref/codebook.py:9-12)
+ *   W_inner  fp16 [in][out] row-major; y = xh @ W_inner
+ * fp16 buffers are passed as uint16_t* (bit patterns).
+ */
+#ifndef EXL3_HIP_H
+#define EXL3_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EXL3_OK 0
+#define EXL3_E_BAD_K (-1)         /* K outside 1..8 */
+#define EXL3_E_BAD_CODEBOOK (-2)  /* cb outside 0..2 */
+#define EXL3_E_BAD_SHAPE (-3)     /* sizes not multiples of 16 / 128, slice out of range, rows out of range */
+#define EXL3_E_NULL_POINTER (-4)  /* a required pointer is NULL */
+#define EXL3_E_WORKSPACE (-5)     /* workspace smaller than exl3_workspace_bytes() reports */
+#define EXL3_E_LAUNCH (-6)        /* hipGetLastError() was not hipSuccess after a launch */
+#define EXL3_E_BAD_INDEX (-7)     /* tile_sub / expert index table inconsistent */
+#define EXL3_E_UNSUPPORTED (-8)   /* valid request this build has no kernel for */
+
+/* Library version (major*10000 + minor*100 + patch). */
+int exl3_version(void);
+
+/* Human-readable text for a status code; never NULL. */
+const char *exl3_status_string(int status);
+
+/* Largest row count the small-batch kernel (exl3_gemv) accepts per call. */
+int exl3_gemv_max_rows(void);
+
+/*
+ * Trellis -> fp16 W_inner for a slice of tile columns.
+ * Replaces decode_full_mlx (ponyexl3/mlx/gemv_metal.py:717-743) and the CPU
+ * decode_packed_trellis (ponyexl3/ref/decode.py:32-81). Bit-exact with both.
+ *   w_out   fp16 [16*in_tiles][16*tn_count] row-major
+ */
+int exl3_decode_full(const uint16_t *trellis, int in_tiles, int out_tiles, int K, int cb,
+                     int tn_offset, int tn_count, uint16_t *w_out, void *stream);
+
+/*
+ * Input-side Hadamard-128 with per-channel multipliers, fp32 butterflies:
+ *   xh[r][s][:] = fp16( H128/sqrt(128) applied per 128-block to (x[r][:] * suh[s][:]) )
+ * Replaces EXL3LayerRuntime.prepare_xh (ponyexl3/mlx/layer_state.py:133-136),
+ * the stacked-suh _fused_prep (ponyexl3/mlx/exl3_fused.py:44-60) and the
+ * pre_scale half of had_r_128 (ponyexl3/ref/hadamard.py:50-80, used at
+ * ponyexl3/ref/forward.py:34).
+ *   x     fp16 [rows][n]
+ *   suh   fp16 [n_sub][n], or NULL (then n_sub must be 1 and no multiply happens)
+ *   xh    fp16 [rows][n_sub][n]
+ */
+int exl3_had128_pre(const uint16_t *x, int rows, int n, const uint16_t *suh, int n_sub,
+                    uint16_t *xh, void *stream);
+
+/*
+ * Output-side Hadamard-128: optional split-K reduction, the fp16 cast of the
+ * matmul result, the transform, svh and bias:
+ *   t   = fp16( sum_{i < n_sum} y[i][r][:] )      (ponyexl3/ref/forward.py:41)
+ *   out = fp16( had128(t) * svh ) (+ bias, fp16 add)  (ponyexl3/ref/forward.py:42-45)
+ * Replaces EXL3LayerRuntime.finish_y (ponyexl3/mlx/layer_state.py:138-141),
+ * _fused_finish (ponyexl3/mlx/exl3_fused.py:63-76) and the partial-sum
+ * reduction of ponyexl3/mlx/gemv_metal.py:1454-1457. Slices are added in index
+ * order, so the result is deterministic.
+ *   y           fp32 [n_sum][rows][n] (y_is_fp32 = 1, slice stride sum_stride
+ *               elements) or fp16 [rows][n] (y_is_fp32 = 0, n_sum must be 1)
+ *   svh, bias   fp16 [n] or NULL
+ *   out         fp16 [rows][n]; may alias y when y is fp16
+ */
+int exl3_had128_post(const void *y, int y_is_fp32, int n_sum, size_t sum_stride, int rows, int n,
+                     const uint16_t *svh, const uint16_t *bias, uint16_t *out, void *stream);
+
+/*
+ * Small-batch fused trellis-decode GEMV/GEMM: y[m] = xh[m, sub(g)] @ W_inner,
+ * fp32 accumulation, rows <= exl3_gemv_max_rows().
+ * Replaces inner_gemv_mlx / inner_gemm_mlx / inner_gem_fused_mlx
+ * (ponyexl3/mlx/gemv_metal.py:1495-1515, 1481-1492) including the split-K
+ * chooser (:1405-1414) and the host-side partial sum (:1454-1457).
+ *
+ *   xh          fp16 [rows][n_sub][in] rotated activations
+ *   group_sub   int32 [out_tiles/8] or NULL: which of the n_sub activation rows
+ *               the 128-column group g multiplies (tile_sub of
+ *               ponyexl3/mlx/exl3_fused.py:107-125 at 128-column granularity)
+ *   group_tile  int32 [n_groups] or NULL: first tile column of each 128-column
+ *               group inside the trellis (tile_map of
+ *               ponyexl3/mlx/exl3_moe.py:139-171 at 128-column granularity);
+ *               NULL = groups 0..out_tiles/8-1 in order
+ *   n_groups    number of 128-column output groups produced (out = 128*n_groups)
+ *   y_out       fp32 [rows][128*n_groups]; partial sums are reduced in a fixed
+ *               order, so results are run-to-run deterministic
+ *   workspace   device scratch of at least exl3_gemv_workspace_bytes(...)
+ */
+int exl3_gemv(const uint16_t *xh, int rows, int n_sub, const uint16_t *trellis, int in_tiles,
+              int out_tiles, int K, int cb, const int32_t *group_sub, const int32_t *group_tile,
+              int n_groups, float *y_out, void *workspace, size_t workspace_bytes, void *stream);
+
+size_t exl3_gemv_workspace_bytes(int rows, int in_tiles, int n_groups);
+
+/*
+ * Prefill GEMM: y = xh @ W_inner for rows > exl3_gemv_max_rows(), trellis tiles
+ * decoded into LDS and contracted on fp16 MFMA with fp32 accumulation.
+ * Replaces the rows > 16 branches of EXL3Linear.__call__
+ * (ponyexl3/mlx/exl3_linear.py:137-161: staged fused GEMM, decode_full + matmul,
+ * striped matmul).
+ *   xh      fp16 [rows][ldx] (ldx >= in, elements)
+ *   y_out   fp16 [rows][ldy] written at column offset 0 (ldy >= out); the fp32
+ *           accumulator is rounded once (the cast at ponyexl3/ref/forward.py:41)
+ */
+int exl3_gemm(const uint16_t *xh, int rows, size_t ldx, const uint16_t *trellis, int in_tiles,
+              int out_tiles, int K, int cb, int tn_offset, int tn_count, uint16_t *y_out,
+              size_t ldy, void *stream);
+
+/*
+ * Whole layer forward (ponyexl3/ref/forward.py:14-49, EXL3Linear.__call__ at
+ * ponyexl3/mlx/exl3_linear.py:98-165, FusedEXL3Group.forward_all at
+ * ponyexl3/mlx/exl3_fused.py:136-202):
+ *   xh = fp16(had(x * suh_s)); y = fp16(xh @ W); y = fp16(had(y) * svh) (+ bias)
+ *   x        fp16 [rows][in]
+ *   suh      fp16 [n_sub][in] or NULL (n_sub = 1 for a plain layer)
+ *   svh      fp16 [out] or NULL
+ *   group_sub int32 [out/128] or NULL (required when n_sub > 1)
+ *   y        fp16 [rows][out]
+ *   workspace at least exl3_linear_workspace_bytes(rows, in, out, n_sub)
+ */
+int exl3_linear_forward(const uint16_t *x, int rows, const uint16_t *trellis, int in_tiles,
+                        int out_tiles, int K, int cb, const uint16_t *suh, int n_sub,
+                        const int32_t *group_sub, const uint16_t *svh, const uint16_t *bias,
+                        uint16_t *y, void *workspace, size_t workspace_bytes, void *stream);
+
+size_t exl3_linear_workspace_bytes(int rows, int in_features, int out_features, int n_sub);
+
+/*
+ * Routed MoE expert chain for rows <= 8 tokens (EXL3SwitchGLU.__call__,
+ * ponyexl3/mlx/exl3_moe.py:770-787; unfused definition :648-682):
+ * per slot (token t, expert e = indices[t][s]):
+ *   g = L_gate,e(x_t); u = L_up,e(x_t); h = fp16(act(g) * u); y = L_down,e(h)
+ *   gu_trellis  uint16 [D/16][E*2*H/16][16K], tile columns laid out
+ *               [all experts' gate | all experts' up] (ponyexl3/mlx/model.py:96-122)
+ *   gu_suh      fp16 [E][2][D];   gu_svh fp16 [E][2*H]
+ *   dn_trellis  uint16 [H/16][E*D/16][16K]
+ *   dn_suh      fp16 [E][H];      dn_svh fp16 [E][D]
+ *   x           fp16 [tokens][D]; indices int32 [tokens][top_k]
+ *   activation  0 = silu (SwiGLU), 1 = tanh-gelu (GeGLU) (ponyexl3/mlx/exl3_moe.py:62-75)
+ *   y           fp16 [tokens][top_k][D]
+ *   workspace   at least exl3_moe_workspace_bytes(tokens, top_k, D, H)
+ * Only the selected experts' trellis blocks are read.
+ */
+int exl3_moe_forward(const uint16_t *x, int tokens, const int32_t *indices, int top_k,
+                     const uint16_t *gu_trellis, const uint16_t *gu_suh, const uint16_t *gu_svh,
+                     const uint16_t *dn_trellis, const uint16_t *dn_suh, const uint16_t *dn_svh,
+                     int num_experts, int D, int H, int K, int cb, int activation, uint16_t *y,
+                     void *workspace, size_t workspace_bytes, void *stream);
+
+size_t exl3_moe_workspace_bytes(int tokens, int top_k, int D, int H);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* EXL3_HIP_H */

@@ -1,0 +1,88 @@
+"""ctypes binding of libexl3_hip.so, the C-ABI library declared in include/exl3_hip.h.
+
+The library is the only compute path of this package: if it has not been built
+(``python -m ponyexl3_amd.build``) loading fails with an error instead of
+falling back to anything else.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "libexl3_hip.so")
+
+EXL3_OK = 0
+EXL3_E_BAD_K = -1
+EXL3_E_BAD_CODEBOOK = -2
+EXL3_E_BAD_SHAPE = -3
+EXL3_E_NULL_POINTER = -4
+EXL3_E_WORKSPACE = -5
+EXL3_E_LAUNCH = -6
+EXL3_E_BAD_INDEX = -7
+EXL3_E_UNSUPPORTED = -8
+
+_vp = ctypes.c_void_p
+_i = ctypes.c_int
+_sz = ctypes.c_size_t
+
+# name -> (restype, argtypes); mirrors include/exl3_hip.h one to one
+PROTOTYPES = {
+    "exl3_version": (_i, []),
+    "exl3_status_string": (ctypes.c_char_p, [_i]),
+    "exl3_gemv_max_rows": (_i, []),
+    "exl3_decode_full": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _vp]),
+    "exl3_had128_pre": (_i, [_vp, _i, _i, _vp, _i, _vp, _vp]),
+    "exl3_had128_post": (_i, [_vp, _i, _i, _sz, _i, _i, _vp, _vp, _vp, _vp]),
+    "exl3_gemv": (_i, [_vp, _i, _i, _vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _sz, _vp]),
+    "exl3_gemv_workspace_bytes": (_sz, [_i, _i, _i]),
+    "exl3_gemm": (_i, [_vp, _i, _sz, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
+    "exl3_linear_forward": (
+        _i,
+        [_vp, _i, _vp, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _sz, _vp],
+    ),
+    "exl3_linear_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "exl3_moe_forward": (
+        _i,
+        [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _sz, _vp],
+    ),
+    "exl3_moe_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load libexl3_hip.so (after torch, so both share one HIP runtime)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build the HIP kernels first with "
+                "`python -m ponyexl3_amd.build` (there is no fallback path)"
+            )
+        import torch  # noqa: F401  (loads libamdhip64 before our library resolves it)
+
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in PROTOTYPES.items():
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = lib
+    return _lib
+
+
+def status_string(status: int) -> str:
+    return load().exl3_status_string(int(status)).decode()
+
+
+def check(status: int, what: str) -> None:
+    """Raise like the reference's host wrappers do: ValueError for argument
+    errors found before launch, RuntimeError if a launch itself failed."""
+    if status == EXL3_OK:
+        return
+    msg = f"{what}: {status_string(status)} (status {status})"
+    if status == EXL3_E_LAUNCH:
+        raise RuntimeError(msg)
+    raise ValueError(msg)

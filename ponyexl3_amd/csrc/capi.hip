@@ -1,0 +1,97 @@
+// Composite C-ABI entry points: status text and the whole-layer forward that
+// chains the Hadamard, GEMV/GEMM and finishing kernels on one stream.
+#include "exl3_device.hpp"
+#include "exl3_host.hpp"
+
+namespace exl3 {
+
+// Workspace layout of exl3_linear_forward:
+//   [0, xh_bytes)            xh  fp16 [rows][n_sub][in]
+//   [xh_bytes, ...)          rows <= kGemvMaxRows: fp32 split-K partials
+//                            otherwise:            fp16 y [rows][out]
+struct LinearWorkspace {
+    size_t xh_bytes;
+    size_t second_bytes;
+    size_t total() const { return xh_bytes + second_bytes; }
+};
+
+static LinearWorkspace linear_workspace(int rows, int in_features, int out_features, int n_sub) {
+    LinearWorkspace w{};
+    w.xh_bytes = align_up((size_t)rows * n_sub * in_features * 2, 256);
+    if (rows <= kGemvMaxRows) {
+        const GemvPlan plan = plan_gemv(rows, in_features / 16, out_features / 128);
+        w.second_bytes = (size_t)plan.n_splits * rows * out_features * sizeof(float);
+    } else {
+        w.second_bytes = (size_t)rows * out_features * 2;
+    }
+    w.second_bytes = align_up(w.second_bytes, 256);
+    return w;
+}
+
+}  // namespace exl3
+
+EXL3_EXPORT int exl3_version(void) { return 100; }
+
+EXL3_EXPORT const char* exl3_status_string(int status) {
+    switch (status) {
+        case EXL3_OK: return "ok";
+        case EXL3_E_BAD_K: return "K must be in [1, 8]";
+        case EXL3_E_BAD_CODEBOOK: return "codebook id must be 0 (3INST), 1 (MCG) or 2 (MUL1)";
+        case EXL3_E_BAD_SHAPE: return "invalid shape, slice, row count or alignment";
+        case EXL3_E_NULL_POINTER: return "a required pointer is NULL";
+        case EXL3_E_WORKSPACE: return "workspace too small";
+        case EXL3_E_LAUNCH: return "HIP kernel launch failed";
+        case EXL3_E_BAD_INDEX: return "inconsistent group/expert index table";
+        case EXL3_E_UNSUPPORTED: return "no kernel for this request";
+        default: return "unknown status";
+    }
+}
+
+EXL3_EXPORT size_t exl3_linear_workspace_bytes(int rows, int in_features, int out_features,
+                                               int n_sub) {
+    if (rows < 1 || in_features < 128 || out_features < 128 || n_sub < 1) return 0;
+    return exl3::linear_workspace(rows, in_features, out_features, n_sub).total();
+}
+
+EXL3_EXPORT int exl3_linear_forward(const uint16_t* x, int rows, const uint16_t* trellis,
+                                    int in_tiles, int out_tiles, int K, int cb,
+                                    const uint16_t* suh, int n_sub, const int32_t* group_sub,
+                                    const uint16_t* svh, const uint16_t* bias, uint16_t* y,
+                                    void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace exl3;
+    if (int rc = check_k_cb(K, cb)) return rc;
+    if (!x || !trellis || !y || !workspace) return EXL3_E_NULL_POINTER;
+    if (rows < 1 || in_tiles < 8 || out_tiles < 8 || in_tiles % 8 || out_tiles % 8 || n_sub < 1)
+        return EXL3_E_BAD_SHAPE;  // Hadamard-128 needs multiples of 128 (ref/hadamard.py:67-68)
+    if (n_sub > 1 && (!group_sub || !suh)) return EXL3_E_BAD_INDEX;
+    const int in_features = in_tiles * 16, out_features = out_tiles * 16;
+    const LinearWorkspace ws = linear_workspace(rows, in_features, out_features, n_sub);
+    if (workspace_bytes < ws.total()) return EXL3_E_WORKSPACE;
+    hipStream_t s = as_stream(stream);
+    uint16_t* xh = reinterpret_cast<uint16_t*>(workspace);
+    char* second = reinterpret_cast<char*>(workspace) + ws.xh_bytes;
+
+    if (int rc = launch_had_pre(x, rows, in_features, suh, n_sub, xh, s)) return rc;
+
+    if (rows <= kGemvMaxRows) {
+        const int n_groups = out_tiles / 8;
+        const GemvPlan plan = plan_gemv(rows, in_tiles, n_groups);
+        float* partial = reinterpret_cast<float*>(second);
+        if (int rc = launch_gemv_partials(xh, rows, n_sub, trellis, in_tiles, out_tiles, K, cb,
+                                          group_sub, nullptr, n_groups, partial, plan, s))
+            return rc;
+        return launch_had_post(partial, 1, plan.n_splits, (size_t)rows * out_features, rows,
+                               out_features, svh, bias, y, s);
+    }
+
+    // Prefill: one GEMM per run of 128-column groups that share an activation row.
+    uint16_t* ytmp = reinterpret_cast<uint16_t*>(second);
+    if (n_sub == 1) {
+        if (int rc = launch_gemm(xh, rows, (size_t)in_features, trellis, in_tiles, out_tiles, K, cb,
+                                 0, out_tiles, ytmp, (size_t)out_features, s))
+            return rc;
+    } else {
+        return EXL3_E_UNSUPPORTED;  // fused groups run their members one by one on the host side
+    }
+    return launch_had_post(ytmp, 0, 1, 0, rows, out_features, svh, bias, y, s);
+}

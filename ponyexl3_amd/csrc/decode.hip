@@ -1,0 +1,84 @@
+// exl3_decode_full: packed trellis -> fp16 W_inner (in, out), bit-exact with
+// ponyexl3/ref/decode.py:32-81.
+//
+// One wavefront decodes the 8 tiles (tk, tn0..tn0+7): its 64 lanes read 256*K
+// contiguous bytes, each lane decodes 32 codewords in registers, the 16x128
+// block is transposed through LDS and written as 16-byte rows.
+#include "exl3_device.hpp"
+#include "exl3_host.hpp"
+
+namespace exl3 {
+
+constexpr int kDecPad = 8;  // halfs of padding per staged row (keeps 16 B alignment)
+
+template <int K, int CB>
+__global__ __launch_bounds__(256) void decode_full_kernel(const uint32_t* __restrict__ trellis,
+                                                          half_t* __restrict__ w_out, int in_tiles,
+                                                          int out_tiles, int tn_offset,
+                                                          int tn_count) {
+    __shared__ __attribute__((aligned(16))) half_t stage[4][16][128 + kDecPad];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int groups = (tn_count + 7) >> 3;
+    const long long wid = (long long)blockIdx.x * 4 + wave;
+    const bool active = wid < (long long)in_tiles * groups;
+    const int g = active ? (int)(wid % groups) : 0;
+    const int tk = active ? (int)(wid / groups) : 0;
+    const int tile_local = g * 8 + (lane >> 3);
+    const bool valid = active && tile_local < tn_count;
+    // lanes of a tile past the slice re-read the last valid tile (never stored)
+    const int tn = tn_offset + (valid ? tile_local : tn_count - 1);
+    const uint32_t* p = trellis + ((size_t)tk * out_tiles + tn) * (8 * K) + (lane & 7) * K;
+    uint32_t own[K];
+#pragma unroll
+    for (int i = 0; i < K; i++) own[i] = p[i];
+    const LaneWords<K> lw = finish_lane_words<K>(own, lane);
+    half2_t wp[16];
+    decode_lane<K, CB>(lw, wp);
+    const int c0 = (lane >> 3) * 16 + (lane & 7);
+#pragma unroll
+    for (int cs = 0; cs < 2; cs++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            stage[wave][2 * j][c0 + 8 * cs] = wp[8 * cs + j].x;
+            stage[wave][2 * j + 1][c0 + 8 * cs] = wp[8 * cs + j].y;
+        }
+    __syncthreads();
+    if (!active) return;
+    const size_t ld = (size_t)tn_count * 16;
+#pragma unroll
+    for (int pass = 0; pass < 4; pass++) {
+        const int row = pass * 4 + (lane >> 4);
+        const int chunk = lane & 15;  // 8 halfs each; two chunks per tile
+        if (g * 8 + (chunk >> 1) < tn_count) {
+            const uint4_t v = *reinterpret_cast<const uint4_t*>(&stage[wave][row][chunk * 8]);
+            *reinterpret_cast<uint4_t*>(w_out + ((size_t)tk * 16 + row) * ld + (size_t)g * 128 +
+                                        chunk * 8) = v;
+        }
+    }
+}
+
+}  // namespace exl3
+
+EXL3_EXPORT int exl3_decode_full(const uint16_t* trellis, int in_tiles, int out_tiles, int K,
+                                 int cb, int tn_offset, int tn_count, uint16_t* w_out,
+                                 void* stream) {
+    using namespace exl3;
+    if (int rc = check_k_cb(K, cb)) return rc;
+    if (!trellis || !w_out) return EXL3_E_NULL_POINTER;
+    if (in_tiles < 0 || out_tiles < 0 || tn_offset < 0 || tn_count < 0 ||
+        tn_offset + tn_count > out_tiles)
+        return EXL3_E_BAD_SHAPE;
+    if (in_tiles == 0 || tn_count == 0) return EXL3_OK;
+    if ((reinterpret_cast<uintptr_t>(w_out) & 15) || (reinterpret_cast<uintptr_t>(trellis) & 3))
+        return EXL3_E_BAD_SHAPE;
+    const long long waves = (long long)in_tiles * ((tn_count + 7) / 8);
+    const long long grid = (waves + 3) / 4;
+    if (grid > 0x7FFFFFFFLL) return EXL3_E_BAD_SHAPE;
+    return dispatch_k_cb(K, cb, [&](auto k, auto c) {
+        decode_full_kernel<k.value, c.value><<<dim3((unsigned)grid), dim3(256), 0, as_stream(stream)>>>(
+            reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<half_t*>(w_out), in_tiles,
+            out_tiles, tn_offset, tn_count);
+        return launch_status();
+    });
+}

@@ -1,0 +1,161 @@
+// Device-side building blocks shared by every EXL3 kernel: fp16 helpers, the
+// procedural codebooks and the per-lane view of a packed trellis tile.
+//
+// Written for gfx950 (CDNA4) only: 64-wide wavefronts, v_bitop3_b32,
+// v_dot2_f32_f16 and the fp16 MFMA family are assumed to exist.
+//
+// Bitstream facts used throughout (reference: ponyexl3/ref/trellis.py:105-141):
+//   * a tile is a circular stream of 256*K bits stored as 8*K little-endian
+//     uint32 words; stream bit b is bit 31-(b%32) of word b/32;
+//   * codeword c (0..255) is the 16 stream bits that end (exclusive) at bit
+//     (c+1)*K, most significant bit first.
+// Tile order facts (reference: ponyexl3/ref/perm.py:8-25): codewords 4l..4l+3
+// (l = 0..63) all belong to output column (l>>3) + 8*(l&1) and to input rows
+// {2q, 2q+1, 2q+8, 2q+9} with q = (l>>1)&3.
+//
+// Lane view: one tile is handled by 8 consecutive lanes. Lane u (0..7) owns
+// codewords 32u..32u+31, whose fresh bits are the K dwords [u*K, (u+1)*K) of the
+// tile, plus the last 16-K bits of the dword before them (the last dword of the
+// tile for u = 0: the stream is circular). Those 32 codewords are the two output
+// columns u and u+8 across all 16 input rows, so a lane can accumulate two
+// output columns without ever exchanging data with another lane.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace exl3 {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+constexpr int kLanesPerTile = 8;    // lanes that share one 16x16 tile
+constexpr int kTilesPerWave = 8;    // tiles covered by one wave-wide load
+constexpr int kColsPerGroup = 128;  // output columns of one wave-wide load
+
+template <int Begin, int End, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (Begin < End) {
+        f(std::integral_constant<int, Begin>{});
+        static_for<Begin + 1, End>(f);
+    }
+}
+
+__device__ __forceinline__ half_t bits_to_half(uint16_t b) { return __builtin_bit_cast(half_t, b); }
+__device__ __forceinline__ uint16_t half_to_bits(half_t h) { return __builtin_bit_cast(uint16_t, h); }
+__device__ __forceinline__ half2_t bits_to_half2(uint32_t b) { return __builtin_bit_cast(half2_t, b); }
+__device__ __forceinline__ uint32_t half2_to_bits(half2_t h) { return __builtin_bit_cast(uint32_t, h); }
+
+// Codebook ids as in ponyexl3/ref/codebook.py:9-12.
+enum : int { CB_3INST = 0, CB_MCG = 1, CB_MUL1 = 2 };
+
+// One codeword (value < 65536) -> one fp16 weight, bit-exact with
+// ponyexl3/ref/codebook.py:66-91.
+//
+// 3INST / MCG: x = cw*M + A (mod 2^32); x = (x & 0x8FFF8FFF) ^ 0x3B603B60; the
+// result is the fp16 sum of the two halves of x (one rounding). The 32-bit
+// product is built from two 16x16 multiplies (full rate) instead of one
+// v_mul_lo_u32 (quarter rate): cw*M = cw*Mlo + ((cw*Mhi) << 16) (mod 2^32).
+//
+// MUL1: x = cw*0x83DCD12D; h = 1024 + (sum of the four bytes of x);
+// result = fp16(h * K_INV + K_BIAS). h*K_INV + K_BIAS is an integer multiple of
+// 2^-18 below 2^4, hence exact in fp32, so the single fp32->fp16 conversion is
+// the only rounding (the reference rounds once from double).
+template <int CB>
+__device__ __forceinline__ half_t decode_cw(uint32_t cw) {
+    if constexpr (CB == CB_MUL1) {
+        const uint32_t x = cw * 0x83DCD12Du;
+        const uint32_t s = __builtin_amdgcn_sad_u8(x, 0u, 1024u);
+        const float v = __builtin_fmaf((float)s, 0.00676727294921875f, -10.3828125f);
+        return (half_t)v;
+    } else {
+        constexpr uint32_t M = (CB == CB_3INST) ? 89226354u : 0xCBAC1FEDu;
+        constexpr uint32_t A = (CB == CB_3INST) ? 64248484u : 0u;
+        const uint32_t lo = cw * (M & 0xFFFFu) + A;
+        const uint32_t hi = cw * (M >> 16);
+        uint32_t x = lo + (hi << 16);
+        x = (x & 0x8FFF8FFFu) ^ 0x3B603B60u;
+        return bits_to_half((uint16_t)(x & 0xFFFFu)) + bits_to_half((uint16_t)(x >> 16));
+    }
+}
+
+// The K+1 dwords a lane needs for its 32 codewords: w[0] is the dword that
+// precedes the lane's own K dwords (already wrapped), w[1..K] are its own.
+template <int K>
+struct LaneWords {
+    uint32_t w[K + 1];
+};
+
+// Codeword N (0..31) of a lane. Bits are numbered MSB-first from the start of
+// w[0]; codeword N ends (exclusive) at bit 32 + (N+1)*K.
+template <int K, int N>
+__device__ __forceinline__ uint32_t lane_codeword(const LaneWords<K>& lw) {
+    constexpr int end = 32 + (N + 1) * K;
+    constexpr int wi = (end - 1) / 32;
+    constexpr int sh = 32 * (wi + 1) - end;
+    if constexpr (sh + 16 <= 32) {
+        return (lw.w[wi] >> sh) & 0xFFFFu;
+    } else {
+        const uint64_t pair = ((uint64_t)lw.w[wi - 1] << 32) | lw.w[wi];
+        return (uint32_t)(pair >> sh) & 0xFFFFu;
+    }
+}
+
+// Where codeword N of a lane sits inside the 16x16 tile:
+//   column = u + 8*col_sel(N), row = tile_row(N).
+__host__ __device__ constexpr int cw_col_sel(int n) { return (n >> 2) & 1; }
+__host__ __device__ constexpr int cw_row(int n) {
+    return 2 * ((n >> 3) & 3) + (n & 1) + 8 * ((n >> 1) & 1);
+}
+
+// Loads the K dwords of lane `lane` for the 8 tiles that start at dword
+// `base` (tile tn0 of row tk) and fetches the preceding dword from the
+// neighbouring lane (lane u-1 of the same tile, u = 0 wraps to u = 7).
+template <int K>
+__device__ __forceinline__ void load_lane_words(const uint32_t* __restrict__ base, int lane,
+                                                uint32_t (&own)[K]) {
+    const uint32_t* p = base + lane * K;
+#pragma unroll
+    for (int i = 0; i < K; i++) own[i] = p[i];
+}
+
+template <int K>
+__device__ __forceinline__ LaneWords<K> finish_lane_words(const uint32_t (&own)[K], int lane) {
+    LaneWords<K> lw;
+    const int src = (lane & ~7) | ((lane + 7) & 7);
+    lw.w[0] = (uint32_t)__shfl((int)own[K - 1], src, kWave);
+#pragma unroll
+    for (int i = 0; i < K; i++) lw.w[i + 1] = own[i];
+    return lw;
+}
+
+// Decodes the lane's 32 codewords into 16 half2 pairs.
+// pair index p = 8*col_sel + q + 4*hi where the pair holds input rows
+// (2q + 8*hi, 2q + 8*hi + 1) of column u + 8*col_sel, i.e. pair j of a column
+// multiplies x[2j], x[2j+1] with j = q + 4*hi.
+template <int K, int CB>
+__device__ __forceinline__ void decode_lane(const LaneWords<K>& lw, half2_t (&wp)[16]) {
+    static_for<0, 16>([&](auto pi) {
+        constexpr int n = 2 * pi.value;  // even codeword of the pair
+        constexpr int cs = cw_col_sel(n);
+        constexpr int j = cw_row(n) >> 1;  // x pair index
+        half2_t v;
+        v.x = decode_cw<CB>(lane_codeword<K, n>(lw));
+        v.y = decode_cw<CB>(lane_codeword<K, n + 1>(lw));
+        wp[8 * cs + j] = v;
+    });
+}
+
+__device__ __forceinline__ float dot2(half2_t a, half2_t b, float c) {
+    return __builtin_amdgcn_fdot2(a, b, c, false);
+}
+
+}  // namespace exl3

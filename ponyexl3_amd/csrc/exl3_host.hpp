@@ -1,0 +1,79 @@
+// Host-side plumbing shared by the translation units of libexl3_hip.so:
+// argument checks, (K, codebook) template dispatch and the internal launchers
+// that the composite entry points (exl3_linear_forward, exl3_moe_forward) chain.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/exl3_hip.h"
+
+#define EXL3_EXPORT extern "C" __attribute__((visibility("default")))
+
+namespace exl3 {
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline int launch_status() { return hipGetLastError() == hipSuccess ? EXL3_OK : EXL3_E_LAUNCH; }
+
+inline int check_k_cb(int K, int cb) {
+    if (K < 1 || K > 8) return EXL3_E_BAD_K;
+    if (cb < 0 || cb > 2) return EXL3_E_BAD_CODEBOOK;
+    return EXL3_OK;
+}
+
+// Calls f(integral_constant<int,K>, integral_constant<int,CB>) for runtime K, cb.
+template <typename F>
+inline int dispatch_k_cb(int K, int cb, F&& f) {
+#define EXL3_CASE_CB(KV)                                                                   \
+    switch (cb) {                                                                          \
+        case 0: return f(std::integral_constant<int, KV>{}, std::integral_constant<int, 0>{}); \
+        case 1: return f(std::integral_constant<int, KV>{}, std::integral_constant<int, 1>{}); \
+        case 2: return f(std::integral_constant<int, KV>{}, std::integral_constant<int, 2>{}); \
+        default: return EXL3_E_BAD_CODEBOOK;                                               \
+    }
+    switch (K) {
+        case 1: EXL3_CASE_CB(1)
+        case 2: EXL3_CASE_CB(2)
+        case 3: EXL3_CASE_CB(3)
+        case 4: EXL3_CASE_CB(4)
+        case 5: EXL3_CASE_CB(5)
+        case 6: EXL3_CASE_CB(6)
+        case 7: EXL3_CASE_CB(7)
+        case 8: EXL3_CASE_CB(8)
+        default: return EXL3_E_BAD_K;
+    }
+#undef EXL3_CASE_CB
+}
+
+constexpr int kGemvMaxRows = 8;
+
+// Split-K plan of the small-batch kernel: the tile rows [0, in_tiles) are cut
+// into n_splits ranges of tk_per_split rows; every (128-column group, split)
+// pair is one workgroup.
+struct GemvPlan {
+    int n_splits;
+    int tk_per_split;
+};
+GemvPlan plan_gemv(int rows, int in_tiles, int n_groups);
+
+// partial: fp32 [n_splits][rows][128*n_groups]
+int launch_gemv_partials(const uint16_t* xh, int rows, int n_sub, const uint16_t* trellis,
+                         int in_tiles, int out_tiles, int K, int cb, const int32_t* group_sub,
+                         const int32_t* group_tile, int n_groups, float* partial, GemvPlan plan,
+                         hipStream_t stream);
+
+int launch_had_pre(const uint16_t* x, int rows, int n, const uint16_t* suh, int n_sub,
+                   uint16_t* xh, hipStream_t stream);
+
+int launch_had_post(const void* y, int y_is_fp32, int n_sum, size_t sum_stride, int rows, int n,
+                    const uint16_t* svh, const uint16_t* bias, uint16_t* out, hipStream_t stream);
+
+int launch_gemm(const uint16_t* xh, int rows, size_t ldx, const uint16_t* trellis, int in_tiles,
+                int out_tiles, int K, int cb, int tn_offset, int tn_count, uint16_t* y_out,
+                size_t ldy, hipStream_t stream);
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+}  // namespace exl3

@@ -1,0 +1,262 @@
+// Routed MoE expert chain for a handful of tokens (decode / speculative verify):
+// per slot (token t, expert e) gate and up GEMVs, GLU, down GEMV, each an EXL3
+// linear with its own suh/svh. Only the selected experts' tile columns of the
+// stacked trellises are read: the GEMV kernel is pointed at them through
+// per-group tables built on the device from the routing indices.
+//
+// Launch chain (all on one stream):
+//   1. moe_prep_kernel      rotated activations per (slot, proj) + group tables
+//   2. gemv_kernel          gate/up partial sums, fp32
+//   3. moe_glu_kernel       split reduction, post-Hadamard, svh, GLU, then the
+//                           down projection's input rotation
+//   4. gemv_kernel          down partial sums
+//   5. moe_finish_kernel    split reduction, post-Hadamard, per-expert svh
+//
+// Semantics follow the unfused chain of ponyexl3/mlx/exl3_moe.py:648-682 with
+// the casts of ponyexl3/ref/forward.py:34,41,42; the Metal A2/B2 kernels
+// (ponyexl3/mlx/exl3_moe.py:345-422) are what this replaces.
+#include "exl3_device.hpp"
+#include "exl3_host.hpp"
+
+#pragma clang fp contract(off)
+
+namespace exl3 {
+
+constexpr float kHadScaleMoe = 0.088388347648318440550f;
+
+__device__ __forceinline__ void wht128_moe(float& a, float& b, int lane) {
+    const float s = a + b, d = a - b;
+    a = s;
+    b = d;
+#pragma unroll
+    for (int bit = 0; bit < 6; bit++) {
+        const int mask = 1 << bit;
+        const float pa = __shfl_xor(a, mask, kWave);
+        const float pb = __shfl_xor(b, mask, kWave);
+        const bool upper = (lane & mask) != 0;
+        a = upper ? pa - a : a + pa;
+        b = upper ? pb - b : b + pb;
+    }
+}
+
+// Routing indices come from the caller's device memory; an out-of-range value is
+// clamped so that it can never turn into an out-of-bounds read.
+__device__ __forceinline__ int clamp_expert(int e, int E) { return e < 0 ? 0 : (e >= E ? E - 1 : e); }
+
+// xh_gu[s][p][:] = fp16(had(x[t] * gu_suh[e][p])); also fills the group tables:
+//   gate/up GEMV group (s, p, hg): sub = 2s+p, tile = (p*E + e)*(H/16) + 8*hg
+//   down GEMV group (s, og):       sub = s,    tile = e*(D/16) + 8*og
+__global__ __launch_bounds__(256) void moe_prep_kernel(
+    const half_t* __restrict__ x, const int* __restrict__ indices,
+    const half_t* __restrict__ gu_suh, half_t* __restrict__ xh_gu, int* __restrict__ gu_sub,
+    int* __restrict__ gu_tile, int* __restrict__ dn_sub, int* __restrict__ dn_tile, int slots,
+    int top_k, int E, int D, int H) {
+    const int lane = threadIdx.x & 63;
+    const int dblocks = D >> 7, hblocks = H >> 7;
+    const int wave_id = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int gtid = blockIdx.x * 256 + threadIdx.x;
+    if (gtid < slots * 2 * hblocks) {
+        const int hg = gtid % hblocks, sp = gtid / hblocks;
+        const int e = clamp_expert(indices[sp >> 1], E);
+        gu_sub[gtid] = sp;
+        gu_tile[gtid] = ((sp & 1) * E + e) * (H >> 4) + 8 * hg;
+    }
+    if (gtid < slots * dblocks) {
+        const int og = gtid % dblocks, s = gtid / dblocks;
+        dn_sub[gtid] = s;
+        dn_tile[gtid] = clamp_expert(indices[s], E) * (D >> 4) + 8 * og;
+    }
+    if (wave_id >= slots * 2 * dblocks) return;
+    const int blk = wave_id % dblocks;
+    const int sp = wave_id / dblocks;
+    const int s = sp >> 1, p = sp & 1;
+    const int t = s / top_k;
+    const int e = clamp_expert(indices[s], E);
+    const half2_t xv = *reinterpret_cast<const half2_t*>(x + (size_t)t * D + blk * 128 + 2 * lane);
+    const half2_t sv = *reinterpret_cast<const half2_t*>(gu_suh + ((size_t)e * 2 + p) * D +
+                                                         blk * 128 + 2 * lane);
+    float a = (float)xv.x * (float)sv.x, b = (float)xv.y * (float)sv.y;
+    wht128_moe(a, b, lane);
+    half2_t o;
+    o.x = (half_t)(a * kHadScaleMoe);
+    o.y = (half_t)(b * kHadScaleMoe);
+    *reinterpret_cast<half2_t*>(xh_gu + (size_t)sp * D + blk * 128 + 2 * lane) = o;
+}
+
+__device__ __forceinline__ float glu_act(float g, float u, int activation) {
+    if (activation == 1) {
+        const float t = 0.797884560803f * (g + 0.044715f * g * g * g);
+        return 0.5f * g * (1.0f + tanhf(t)) * u;
+    }
+    return (g / (1.0f + expf(-g))) * u;
+}
+
+// One wave per (slot, 128-block of H): finishes gate and up, applies the GLU and
+// rotates the result for the down projection.
+__global__ __launch_bounds__(256) void moe_glu_kernel(
+    const float* __restrict__ partial, int n_splits, size_t split_stride,
+    const int* __restrict__ indices, const half_t* __restrict__ gu_svh,
+    const half_t* __restrict__ dn_suh, half_t* __restrict__ xh_dn, int slots, int H, int E,
+    int activation) {
+    const int lane = threadIdx.x & 63;
+    const int hblocks = H >> 7;
+    const int wave_id = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (wave_id >= slots * hblocks) return;
+    const int blk = wave_id % hblocks, s = wave_id / hblocks;
+    const int e = clamp_expert(indices[s], E);
+    float v[2][2];
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+        // partial layout: [split][(s*2+p)*H + h]
+        const size_t off = ((size_t)s * 2 + p) * H + blk * 128 + 2 * lane;
+        float2_t acc = *reinterpret_cast<const float2_t*>(partial + off);
+        for (int i = 1; i < n_splits; i++) {
+            const float2_t q = *reinterpret_cast<const float2_t*>(partial + i * split_stride + off);
+            acc.x = acc.x + q.x;
+            acc.y = acc.y + q.y;
+        }
+        float a = (float)(half_t)acc.x, b = (float)(half_t)acc.y;
+        wht128_moe(a, b, lane);
+        const half2_t sv = *reinterpret_cast<const half2_t*>(gu_svh + (size_t)e * 2 * H + p * H +
+                                                             blk * 128 + 2 * lane);
+        v[p][0] = (float)(half_t)(a * kHadScaleMoe * (float)sv.x);
+        v[p][1] = (float)(half_t)(b * kHadScaleMoe * (float)sv.y);
+    }
+    const float h0 = (float)(half_t)glu_act(v[0][0], v[1][0], activation);
+    const float h1 = (float)(half_t)glu_act(v[0][1], v[1][1], activation);
+    const half2_t ds =
+        *reinterpret_cast<const half2_t*>(dn_suh + (size_t)e * H + blk * 128 + 2 * lane);
+    float a = h0 * (float)ds.x, b = h1 * (float)ds.y;
+    wht128_moe(a, b, lane);
+    half2_t o;
+    o.x = (half_t)(a * kHadScaleMoe);
+    o.y = (half_t)(b * kHadScaleMoe);
+    *reinterpret_cast<half2_t*>(xh_dn + (size_t)s * H + blk * 128 + 2 * lane) = o;
+}
+
+__global__ __launch_bounds__(256) void moe_finish_kernel(
+    const float* __restrict__ partial, int n_splits, size_t split_stride,
+    const int* __restrict__ indices, const half_t* __restrict__ dn_svh, half_t* __restrict__ y,
+    int slots, int D, int E) {
+    const int lane = threadIdx.x & 63;
+    const int dblocks = D >> 7;
+    const int wave_id = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (wave_id >= slots * dblocks) return;
+    const int blk = wave_id % dblocks, s = wave_id / dblocks;
+    const int e = clamp_expert(indices[s], E);
+    const size_t off = (size_t)s * D + blk * 128 + 2 * lane;
+    float2_t acc = *reinterpret_cast<const float2_t*>(partial + off);
+    for (int i = 1; i < n_splits; i++) {
+        const float2_t q = *reinterpret_cast<const float2_t*>(partial + i * split_stride + off);
+        acc.x = acc.x + q.x;
+        acc.y = acc.y + q.y;
+    }
+    float a = (float)(half_t)acc.x, b = (float)(half_t)acc.y;
+    wht128_moe(a, b, lane);
+    const half2_t sv =
+        *reinterpret_cast<const half2_t*>(dn_svh + (size_t)e * D + blk * 128 + 2 * lane);
+    half2_t o;
+    o.x = (half_t)(a * kHadScaleMoe * (float)sv.x);
+    o.y = (half_t)(b * kHadScaleMoe * (float)sv.y);
+    *reinterpret_cast<half2_t*>(y + off) = o;
+}
+
+struct MoeWorkspace {
+    size_t xh_gu, xh_dn, tables, part_gu, part_dn;
+    size_t o_xh_gu, o_xh_dn, o_tables, o_part_gu, o_part_dn, total;
+    GemvPlan plan_gu, plan_dn;
+    int g_gu, g_dn;
+};
+
+static MoeWorkspace moe_workspace(int tokens, int top_k, int D, int H) {
+    MoeWorkspace w{};
+    const int slots = tokens * top_k;
+    w.g_gu = slots * 2 * (H / 128);
+    w.g_dn = slots * (D / 128);
+    w.plan_gu = plan_gemv(1, D / 16, w.g_gu);
+    w.plan_dn = plan_gemv(1, H / 16, w.g_dn);
+    w.xh_gu = align_up((size_t)slots * 2 * D * 2, 256);
+    w.xh_dn = align_up((size_t)slots * H * 2, 256);
+    w.tables = align_up((size_t)2 * (w.g_gu + w.g_dn) * sizeof(int), 256);
+    w.part_gu = align_up((size_t)w.plan_gu.n_splits * w.g_gu * 128 * sizeof(float), 256);
+    w.part_dn = align_up((size_t)w.plan_dn.n_splits * w.g_dn * 128 * sizeof(float), 256);
+    w.o_xh_gu = 0;
+    w.o_xh_dn = w.o_xh_gu + w.xh_gu;
+    w.o_tables = w.o_xh_dn + w.xh_dn;
+    w.o_part_gu = w.o_tables + w.tables;
+    w.o_part_dn = w.o_part_gu + w.part_gu;
+    w.total = w.o_part_dn + w.part_dn;
+    return w;
+}
+
+}  // namespace exl3
+
+EXL3_EXPORT size_t exl3_moe_workspace_bytes(int tokens, int top_k, int D, int H) {
+    if (tokens < 1 || top_k < 1 || D < 128 || H < 128 || D % 128 || H % 128) return 0;
+    return exl3::moe_workspace(tokens, top_k, D, H).total;
+}
+
+EXL3_EXPORT int exl3_moe_forward(const uint16_t* x, int tokens, const int32_t* indices, int top_k,
+                                 const uint16_t* gu_trellis, const uint16_t* gu_suh,
+                                 const uint16_t* gu_svh, const uint16_t* dn_trellis,
+                                 const uint16_t* dn_suh, const uint16_t* dn_svh, int num_experts,
+                                 int D, int H, int K, int cb, int activation, uint16_t* y,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace exl3;
+    if (int rc = check_k_cb(K, cb)) return rc;
+    if (!x || !indices || !gu_trellis || !gu_suh || !gu_svh || !dn_trellis || !dn_suh || !dn_svh ||
+        !y || !workspace)
+        return EXL3_E_NULL_POINTER;
+    if (tokens < 1 || top_k < 1 || num_experts < 1 || D < 128 || H < 128 || D % 128 || H % 128 ||
+        (long long)tokens * top_k > 4096)
+        return EXL3_E_BAD_SHAPE;
+    if (activation != 0 && activation != 1) return EXL3_E_UNSUPPORTED;
+    const MoeWorkspace w = moe_workspace(tokens, top_k, D, H);
+    if (workspace_bytes < w.total) return EXL3_E_WORKSPACE;
+    hipStream_t s = as_stream(stream);
+    char* base = reinterpret_cast<char*>(workspace);
+    half_t* xh_gu = reinterpret_cast<half_t*>(base + w.o_xh_gu);
+    half_t* xh_dn = reinterpret_cast<half_t*>(base + w.o_xh_dn);
+    int* gu_sub = reinterpret_cast<int*>(base + w.o_tables);
+    int* gu_tile = gu_sub + w.g_gu;
+    int* dn_sub = gu_tile + w.g_gu;
+    int* dn_tile = dn_sub + w.g_dn;
+    float* part_gu = reinterpret_cast<float*>(base + w.o_part_gu);
+    float* part_dn = reinterpret_cast<float*>(base + w.o_part_dn);
+    const int slots = tokens * top_k;
+
+    {
+        const int waves = slots * 2 * (D / 128);
+        const int threads = waves * 64 > w.g_gu ? waves * 64 : w.g_gu;
+        const int need = threads > w.g_dn ? threads : w.g_dn;
+        moe_prep_kernel<<<dim3((need + 255) / 256), dim3(256), 0, s>>>(
+            reinterpret_cast<const half_t*>(x), indices, reinterpret_cast<const half_t*>(gu_suh),
+            xh_gu, gu_sub, gu_tile, dn_sub, dn_tile, slots, top_k, num_experts, D, H);
+        if (int rc = launch_status()) return rc;
+    }
+    // gate/up: rows = 1, n_sub = 2*slots activation rows, one group per (slot, proj, hg)
+    if (int rc = launch_gemv_partials(reinterpret_cast<const uint16_t*>(xh_gu), 1, slots * 2,
+                                      gu_trellis, D / 16, num_experts * 2 * (H / 16), K, cb,
+                                      gu_sub, gu_tile, w.g_gu, part_gu, w.plan_gu, s))
+        return rc;
+    {
+        const int waves = slots * (H / 128);
+        moe_glu_kernel<<<dim3((waves + 3) / 4), dim3(256), 0, s>>>(
+            part_gu, w.plan_gu.n_splits, (size_t)w.g_gu * 128, indices,
+            reinterpret_cast<const half_t*>(gu_svh), reinterpret_cast<const half_t*>(dn_suh), xh_dn,
+            slots, H, num_experts, activation);
+        if (int rc = launch_status()) return rc;
+    }
+    if (int rc = launch_gemv_partials(reinterpret_cast<const uint16_t*>(xh_dn), 1, slots,
+                                      dn_trellis, H / 16, num_experts * (D / 16), K, cb, dn_sub,
+                                      dn_tile, w.g_dn, part_dn, w.plan_dn, s))
+        return rc;
+    {
+        const int waves = slots * (D / 128);
+        moe_finish_kernel<<<dim3((waves + 3) / 4), dim3(256), 0, s>>>(
+            part_dn, w.plan_dn.n_splits, (size_t)w.g_dn * 128, indices,
+            reinterpret_cast<const half_t*>(dn_svh), reinterpret_cast<half_t*>(y), slots, D,
+            num_experts);
+        return launch_status();
+    }
+}

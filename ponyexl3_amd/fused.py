@@ -1,0 +1,128 @@
+"""Fused sibling groups: several same-K linears that share an input run as one
+launch chain over a concatenated trellis.
+
+Mirrors ``FusedEXL3Group`` / ``FusedEXL3Sibling`` / ``fusable``
+(ponyexl3/mlx/exl3_fused.py:79-228). Members are concatenated along out_tiles,
+``suh`` rows are stacked so each member sees its own rotated activations, and
+``svh`` is concatenated (member out_features are multiples of 128, so an output
+Hadamard block never straddles two members).
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _lib, ops
+from .layer import EXL3Layer, codebook_mode_from_flags, unpack_signs_or_pass
+
+
+def fusable(layers: list[EXL3Layer]) -> bool:
+    first = layers[0]
+    return (
+        len(layers) >= 2
+        and all(l.in_features == first.in_features for l in layers)
+        and all(l.k == first.k for l in layers)
+        and all((l.mcg, l.mul1) == (first.mcg, first.mul1) for l in layers)
+        and all(l.out_features % 128 == 0 for l in layers)
+        and all(l.suh is not None and l.svh is not None for l in layers)
+        and all(l.bias is None for l in layers)
+    )
+
+
+class FusedEXL3Group(torch.nn.Module):
+    """Owner of the concatenated trellis + stacked signs for sibling linears."""
+
+    def __init__(self, layers: list[EXL3Layer], device="cuda"):
+        super().__init__()
+        if not fusable(layers):
+            raise ValueError("layers not fusable: " + ", ".join(l.key for l in layers))
+        for l in layers:
+            l.validate()
+        if layers[0].in_features % 128:
+            raise ValueError("in_features must be a multiple of 128")
+        self._keys = [l.key for l in layers]
+        self._k = int(layers[0].k)
+        self._cb = int(codebook_mode_from_flags(mcg=layers[0].mcg, mul1=layers[0].mul1))
+        self.in_features = layers[0].in_features
+        self._out_features = [l.out_features for l in layers]
+        self._trellis = ops.as_trellis_tensor(
+            np.concatenate([np.asarray(l.trellis).view(np.uint16) for l in layers], axis=1), device
+        )
+        suh = np.stack([unpack_signs_or_pass(l.suh) for l in layers]).astype(np.float16)
+        svh = np.concatenate([unpack_signs_or_pass(l.svh) for l in layers]).astype(np.float16)
+        self._suh_stack = torch.from_numpy(suh).to(device)
+        self._svh_cat = torch.from_numpy(svh).to(device)
+        tile_sub = np.repeat(
+            np.arange(len(layers), dtype=np.uint32), [l.out_features // 16 for l in layers]
+        )
+        self._tile_sub = tile_sub
+        self._group_sub = ops.group_sub_from_tile_sub(tile_sub).to(device)
+        self._cache_x = None
+        self._cache_out = None
+
+    def extra_repr(self) -> str:
+        return f"members={self._keys}, k={self._k}"
+
+    def forward_all(self, x: torch.Tensor) -> tuple[torch.Tensor, ...]:
+        lead = tuple(x.shape[:-1])
+        x2d = x.reshape(-1, self.in_features).to(torch.float16).contiguous()
+        rows = x2d.shape[0]
+        total_out = sum(self._out_features)
+        if rows <= ops.gemv_max_rows():
+            y = ops.linear_forward(
+                x2d, self._trellis, self._k, self._cb, self._suh_stack, self._svh_cat, None,
+                self._group_sub,
+            )
+        else:
+            # prefill: one MFMA GEMM per member over its tile-column range, each
+            # reading its own rotated activations out of the stacked buffer
+            xh = ops.had128_pre(x2d, self._suh_stack)  # (rows, n_sub, in)
+            n_sub = len(self._out_features)
+            yraw = torch.empty((rows, total_out), dtype=torch.float16, device=x2d.device)
+            lib = _lib.load()
+            in_tiles, out_tiles = self.in_features // 16, total_out // 16
+            tn0 = 0
+            for i, n in enumerate(self._out_features):
+                rc = lib.exl3_gemm(
+                    ctypes.c_void_p(xh.data_ptr() + 2 * i * self.in_features), rows,
+                    n_sub * self.in_features, ctypes.c_void_p(self._trellis.data_ptr()),
+                    in_tiles, out_tiles, self._k, self._cb, tn0, n // 16,
+                    ctypes.c_void_p(yraw.data_ptr() + 2 * 16 * tn0), total_out,
+                    ctypes.c_void_p(torch.cuda.current_stream().cuda_stream),
+                )
+                _lib.check(rc, "exl3_gemm")
+                tn0 += n // 16
+            y = ops.had128_post(yraw, self._svh_cat)
+        outs = torch.split(y, self._out_features, dim=-1)
+        return tuple(o.reshape(lead + (n,)) for o, n in zip(outs, self._out_features))
+
+    def cached(self, x: torch.Tensor) -> tuple[torch.Tensor, ...]:
+        if self._cache_out is None or self._cache_x is not x:
+            self._cache_out = self.forward_all(x)
+            self._cache_x = x
+        return self._cache_out
+
+    def sibling(self, idx: int) -> "FusedEXL3Sibling":
+        return FusedEXL3Sibling(self, idx)
+
+
+class FusedEXL3Sibling(torch.nn.Module):
+    """Drop-in replacement for one member linear; delegates to the group and
+    serves from its single-slot input-identity cache."""
+
+    def __init__(self, group: FusedEXL3Group, idx: int):
+        super().__init__()
+        # keep the group out of the module tree: siblings do not own it
+        object.__setattr__(self, "_group", group)
+        self._idx = idx
+        self.in_features = group.in_features
+        self.out_features = group._out_features[idx]
+
+    def extra_repr(self) -> str:
+        return f"{self._group._keys[self._idx]} (member {self._idx})"
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self._group.cached(x)[self._idx]

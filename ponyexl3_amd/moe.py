@@ -1,0 +1,117 @@
+"""Routed MoE experts (stacked EXL3 SwitchGLU) on ROCm tensors.
+
+Mirrors ``EXL3SwitchGLU`` (ponyexl3/mlx/exl3_moe.py:425-457,770-787) and the
+router / weighted sum of ``EXL3MoEBlock`` (ponyexl3/mlx/exl3_moe.py:790-839).
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from . import ops
+from .layer import EXL3Layer, codebook_mode_from_flags, unpack_signs_or_pass
+
+_MOE_ACTIVATIONS = {"silu": 0, "gelu": 1}
+
+
+class EXL3SwitchGLU(torch.nn.Module):
+    """Stacked-expert EXL3 SwitchGLU: ``(x (B,S,D), indices (B,S,kk)) -> (B,S,kk,D)``.
+
+    gu_trellis (D/16, E*2*H/16, 16K) laid out [all experts' gate | all experts' up],
+    gu_suh (E, 2, D), gu_svh (E, 2*H), dn_trellis (H/16, E*D/16, 16K),
+    dn_suh (E, H), dn_svh (E, D)."""
+
+    def __init__(self, *, gu_trellis, gu_suh, gu_svh, dn_trellis, dn_suh, dn_svh, k, cb,
+                 activation: str = "silu"):
+        super().__init__()
+        if activation not in _MOE_ACTIVATIONS:
+            raise ValueError(f"unsupported MoE activation {activation!r}")
+        self._gu_trellis = gu_trellis
+        self._gu_suh = gu_suh
+        self._gu_svh = gu_svh
+        self._dn_trellis = dn_trellis
+        self._dn_suh = dn_suh
+        self._dn_svh = dn_svh
+        self._k = int(k)
+        self._cb = int(cb)
+        self._activation = activation
+        self.num_experts = int(gu_suh.shape[0])
+        self.input_dims = int(gu_suh.shape[2])
+        self.hidden_dims = int(dn_suh.shape[1])
+        E, D, H = self.num_experts, self.input_dims, self.hidden_dims
+        if D % 128 or H % 128:
+            raise ValueError("MoE dims must be multiples of 128")
+        expect = {
+            "gu_trellis": (D // 16, E * 2 * H // 16, 16 * self._k),
+            "gu_suh": (E, 2, D),
+            "gu_svh": (E, 2 * H),
+            "dn_trellis": (H // 16, E * D // 16, 16 * self._k),
+            "dn_suh": (E, H),
+            "dn_svh": (E, D),
+        }
+        for name, shape in expect.items():
+            got = tuple(getattr(self, "_" + name).shape)
+            if got != shape:
+                raise ValueError(f"{name} shape {got} != expected {shape}")
+
+    @classmethod
+    def from_layers(cls, gate: list[EXL3Layer], up: list[EXL3Layer], down: list[EXL3Layer],
+                    activation: str = "silu", device="cuda") -> "EXL3SwitchGLU":
+        """Stack per-expert layers the way the reference's loader does
+        (ponyexl3/mlx/model.py:96-122)."""
+        first = gate[0]
+        for l in gate + up + down:
+            l.validate()
+            if (l.k, l.mcg, l.mul1) != (first.k, first.mcg, first.mul1):
+                raise ValueError("all expert layers must share K and codebook")
+        tr = lambda ls: np.concatenate([np.asarray(l.trellis).view(np.uint16) for l in ls], axis=1)
+        sg = lambda v: unpack_signs_or_pass(v).astype(np.float16)
+        h = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
+        return cls(
+            gu_trellis=ops.as_trellis_tensor(np.concatenate([tr(gate), tr(up)], axis=1), device),
+            gu_suh=h(np.stack([np.stack([sg(g.suh), sg(u.suh)]) for g, u in zip(gate, up)])),
+            gu_svh=h(np.stack([np.concatenate([sg(g.svh), sg(u.svh)]) for g, u in zip(gate, up)])),
+            dn_trellis=ops.as_trellis_tensor(tr(down), device),
+            dn_suh=h(np.stack([sg(d.suh) for d in down])),
+            dn_svh=h(np.stack([sg(d.svh) for d in down])),
+            k=first.k,
+            cb=int(codebook_mode_from_flags(mcg=first.mcg, mul1=first.mul1)),
+            activation=activation,
+        )
+
+    def forward(self, x: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
+        if indices.dim() != 3:
+            raise ValueError("indices must be (B, S, top_k)")
+        B, S, kk = indices.shape
+        R = B * S
+        D = self.input_dims
+        x2d = x.reshape(R, D).to(torch.float16).contiguous()
+        idx = indices.reshape(R, kk).to(torch.int32).contiguous()
+        chunk = max(1, 4096 // kk)
+        outs = []
+        for r0 in range(0, R, chunk):
+            outs.append(
+                ops.moe_forward(
+                    x2d[r0 : r0 + chunk], idx[r0 : r0 + chunk], self._gu_trellis, self._gu_suh,
+                    self._gu_svh, self._dn_trellis, self._dn_suh, self._dn_svh, self._k, self._cb,
+                    _MOE_ACTIVATIONS[self._activation],
+                )
+            )
+        y = outs[0] if len(outs) == 1 else torch.cat(outs, dim=0)
+        return y.reshape(B, S, kk, D)
+
+
+def route_topk(logits: torch.Tensor, top_k: int, norm_topk_prob: bool = True):
+    """softmax (fp32) -> top-k -> optional renormalisation
+    (ponyexl3/mlx/exl3_moe.py:817-821). Returns (indices int32, scores fp32)."""
+    gates = torch.softmax(logits.float(), dim=-1)
+    scores, inds = torch.topk(gates, top_k, dim=-1)
+    if norm_topk_prob:
+        scores = scores / scores.sum(dim=-1, keepdim=True)
+    return inds.to(torch.int32), scores
+
+
+def combine_experts(y: torch.Tensor, scores: torch.Tensor) -> torch.Tensor:
+    """(…, kk, D) x (…, kk) -> (…, D) (ponyexl3/mlx/exl3_moe.py:838-839)."""
+    return (y * scores[..., None].to(y.dtype)).sum(dim=-2)

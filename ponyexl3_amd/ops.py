@@ -1,0 +1,323 @@
+"""Inner operators on torch (ROCm) tensors, thin wrappers over the C ABI.
+
+These mirror the reference's inner operator API
+(``ponyexl3/mlx/gemv_metal.py:717-743,1481-1515`` and
+``ponyexl3/mlx/layer_state.py:133-141``): same names, argument meaning and
+ValueError-before-launch behaviour; arrays are torch tensors on the GPU and
+all launches go to torch's current HIP stream. PyTorch only provides device
+memory and streams here; every result is produced by libexl3_hip.so.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _lib
+
+_workspaces: dict = {}
+
+
+def _check_cuda(t: torch.Tensor, name: str) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise ValueError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (got device {t.device})")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def workspace(device, nbytes: int) -> torch.Tensor:
+    """Per-device scratch buffer shared by all calls on that device (grown on
+    demand). Calls that overlap on different streams of one device would race
+    on it; the reference runs one stream too."""
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+def as_trellis_tensor(trellis, device=None) -> torch.Tensor:
+    """numpy/torch uint16|int16 (in_tiles, out_tiles, 16K) -> int16 GPU tensor
+    holding the same bits."""
+    if isinstance(trellis, np.ndarray):
+        if trellis.dtype not in (np.uint16, np.int16):
+            raise ValueError(f"trellis must be uint16/int16, got {trellis.dtype}")
+        t = torch.from_numpy(np.ascontiguousarray(trellis).view(np.int16))
+    else:
+        t = trellis
+        if t.dtype == torch.uint16:
+            t = t.view(torch.int16)
+        if t.dtype != torch.int16:
+            raise ValueError(f"trellis must be uint16/int16, got {t.dtype}")
+    if device is not None:
+        t = t.to(device)
+    return t.contiguous()
+
+
+def _trellis_dims(trellis: torch.Tensor, k: int):
+    _check_cuda(trellis, "trellis")
+    if trellis.dtype not in (torch.int16, torch.uint16):
+        raise ValueError(f"trellis must be a 16-bit integer tensor, got {trellis.dtype}")
+    if trellis.dim() != 3:
+        raise ValueError("trellis must be 3D (in_tiles, out_tiles, 16*K)")
+    if not 1 <= int(k) <= 8:
+        raise ValueError(f"K must be in [1, 8], got {k}")
+    in_tiles, out_tiles, ps = trellis.shape
+    if ps != 16 * k:
+        raise ValueError(f"packed size {ps} != expected {16 * k} for K={k}")
+    return int(in_tiles), int(out_tiles)
+
+
+def _half(t: torch.Tensor, name: str) -> torch.Tensor:
+    _check_cuda(t, name)
+    if t.dtype != torch.float16:
+        raise ValueError(f"{name} must be float16, got {t.dtype}")
+    return t
+
+
+def decode_full(trellis, k: int, cb: int, tn_offset: int = 0, tn_count: int | None = None):
+    """Trellis -> fp16 W (in, 16*tn_count) (``decode_full_mlx``,
+    ponyexl3/mlx/gemv_metal.py:717-743)."""
+    in_tiles, out_tiles = _trellis_dims(trellis, k)
+    if tn_count is None:
+        tn_count = out_tiles - tn_offset
+    if tn_offset < 0 or tn_count < 0 or tn_offset + tn_count > out_tiles:
+        raise ValueError("slice exceeds output features")
+    w = torch.empty((in_tiles * 16, tn_count * 16), dtype=torch.float16, device=trellis.device)
+    rc = _lib.load().exl3_decode_full(
+        _ptr(trellis), in_tiles, out_tiles, int(k), int(cb), int(tn_offset), int(tn_count),
+        _ptr(w), _stream(),
+    )
+    _lib.check(rc, "exl3_decode_full")
+    return w
+
+
+def had128_pre(x2d: torch.Tensor, suh: torch.Tensor | None):
+    """xh = fp16(had128(x * suh)); suh (in,) or stacked (n_sub, in) -> xh
+    (rows, in) or (rows, n_sub, in). ``EXL3LayerRuntime.prepare_xh`` /
+    ``_fused_prep`` (ponyexl3/mlx/layer_state.py:133-136, exl3_fused.py:44-60)."""
+    _half(x2d, "x")
+    if x2d.dim() != 2:
+        raise ValueError("had128_pre expects 2D input (rows, features)")
+    rows, n = x2d.shape
+    if n % 128 != 0:
+        raise ValueError(f"feature dim {n} not divisible by 128")
+    n_sub = 1
+    stacked = False
+    if suh is not None:
+        _half(suh, "suh")
+        stacked = suh.dim() == 2
+        n_sub = suh.shape[0] if stacked else 1
+        if suh.shape[-1] != n:
+            raise ValueError("suh length does not match the feature dim")
+    shape = (rows, n_sub, n) if stacked else (rows, n)
+    xh = torch.empty(shape, dtype=torch.float16, device=x2d.device)
+    rc = _lib.load().exl3_had128_pre(_ptr(x2d), rows, n, _ptr(suh), n_sub, _ptr(xh), _stream())
+    _lib.check(rc, "exl3_had128_pre")
+    return xh
+
+
+def had128_post(y: torch.Tensor, svh: torch.Tensor | None, bias: torch.Tensor | None = None):
+    """out = fp16(had128(fp16(sum of y slices)) * svh) (+ bias).
+
+    y: fp16 (rows, n), fp32 (rows, n) or fp32 (n_sum, rows, n) split-K partials.
+    ``EXL3LayerRuntime.finish_y`` (ponyexl3/mlx/layer_state.py:138-141)."""
+    _check_cuda(y, "y")
+    if y.dtype == torch.float16:
+        if y.dim() != 2:
+            raise ValueError("fp16 y must be 2D (rows, features)")
+        n_sum, (rows, n), is32 = 1, y.shape, 0
+    elif y.dtype == torch.float32:
+        if y.dim() == 2:
+            n_sum, (rows, n) = 1, y.shape
+        elif y.dim() == 3:
+            n_sum, rows, n = y.shape
+        else:
+            raise ValueError("fp32 y must be (rows, n) or (n_sum, rows, n)")
+        is32 = 1
+    else:
+        raise ValueError(f"y must be float16 or float32, got {y.dtype}")
+    if n % 128 != 0:
+        raise ValueError(f"feature dim {n} not divisible by 128")
+    for name, v in (("svh", svh), ("bias", bias)):
+        if v is not None:
+            _half(v, name)
+            if v.numel() != n:
+                raise ValueError(f"{name} length does not match the feature dim")
+    out = torch.empty((rows, n), dtype=torch.float16, device=y.device)
+    rc = _lib.load().exl3_had128_post(
+        _ptr(y), is32, int(n_sum), rows * n, int(rows), int(n), _ptr(svh), _ptr(bias), _ptr(out),
+        _stream(),
+    )
+    _lib.check(rc, "exl3_had128_post")
+    return out
+
+
+def gemv_max_rows() -> int:
+    return int(_lib.load().exl3_gemv_max_rows())
+
+
+def group_sub_from_tile_sub(tile_sub) -> torch.Tensor:
+    """tile_sub (out_tiles,) -> per-128-column table; every run of 8 tiles must
+    share one member (members have out_features % 128 == 0)."""
+    ts = np.asarray(tile_sub.cpu() if isinstance(tile_sub, torch.Tensor) else tile_sub)
+    ts = ts.astype(np.int64).reshape(-1)
+    if ts.size % 8 != 0:
+        raise ValueError("tile_sub length must be a multiple of 8")
+    g = ts.reshape(-1, 8)
+    if not (g == g[:, :1]).all():
+        raise ValueError("tile_sub must be constant inside each 128-column group")
+    return torch.from_numpy(g[:, 0].astype(np.int32).copy())
+
+
+def inner_gem_fused(xh, trellis, k: int, cb: int, group_sub=None, group_tile=None, n_groups=None):
+    """y (rows, 128*n_groups) fp32 = xh[:, sub(g), :] @ W for rows <= gemv_max_rows().
+
+    xh (rows, n_sub, in) fp16. ``inner_gem_fused_mlx`` /
+    ``_mapped_gemv`` (ponyexl3/mlx/gemv_metal.py:1481-1492, exl3_moe.py:139-171)
+    with tile tables at 128-column granularity."""
+    in_tiles, out_tiles = _trellis_dims(trellis, k)
+    _half(xh, "xh")
+    if xh.dim() != 3:
+        raise ValueError("xh must be (rows, n_sub, in)")
+    rows, n_sub, n_in = xh.shape
+    if n_in != in_tiles * 16:
+        raise ValueError(f"xh features {n_in} != trellis in_features {in_tiles * 16}")
+    if n_in % 128 or out_tiles % 8:
+        raise ValueError("in/out features must be multiples of 128")
+    if not 1 <= rows <= gemv_max_rows():
+        raise ValueError(f"rows must be in [1, {gemv_max_rows()}], got {rows}")
+    if n_groups is None:
+        n_groups = out_tiles // 8 if group_tile is None else int(group_tile.numel())
+    for name, v, need in (("group_sub", group_sub, n_sub > 1), ("group_tile", group_tile, False)):
+        if v is None:
+            if need:
+                raise ValueError(f"{name} is required when n_sub > 1")
+            continue
+        _check_cuda(v, name)
+        if v.dtype != torch.int32 or v.numel() != n_groups:
+            raise ValueError(f"{name} must be int32 with {n_groups} entries")
+    lib = _lib.load()
+    ws_bytes = int(lib.exl3_gemv_workspace_bytes(rows, in_tiles, n_groups))
+    ws = workspace(xh.device, ws_bytes)
+    y = torch.empty((rows, n_groups * 128), dtype=torch.float32, device=xh.device)
+    rc = lib.exl3_gemv(
+        _ptr(xh), rows, n_sub, _ptr(trellis), in_tiles, out_tiles, int(k), int(cb),
+        _ptr(group_sub), _ptr(group_tile), int(n_groups), _ptr(y), _ptr(ws), ws.numel(), _stream(),
+    )
+    _lib.check(rc, "exl3_gemv")
+    return y
+
+
+def inner_gemv(xh, trellis, k: int, cb: int):
+    """(in,) fp16 -> (out,) fp32 (``inner_gemv_mlx``, gemv_metal.py:1495-1505)."""
+    if xh.dim() != 1:
+        raise ValueError("inner_gemv expects a 1D activation vector")
+    return inner_gem_fused(xh.reshape(1, 1, -1), trellis, k, cb).reshape(-1)
+
+
+def inner_gemm(xh, trellis, k: int, cb: int, tn_offset: int = 0, tn_count: int | None = None):
+    """(M, in) fp16 -> (M, out) : fp32 from the small-batch kernel for
+    M <= gemv_max_rows(), fp16 (the oracle's cast of the fp32 accumulator) from
+    the MFMA prefill kernel above that (``inner_gemm_mlx``,
+    gemv_metal.py:1508-1515; exl3_linear.py:137-161)."""
+    in_tiles, out_tiles = _trellis_dims(trellis, k)
+    _half(xh, "xh")
+    if xh.dim() != 2:
+        raise ValueError("inner_gemm expects (M, in)")
+    rows, n_in = xh.shape
+    if n_in != in_tiles * 16:
+        raise ValueError(f"xh features {n_in} != trellis in_features {in_tiles * 16}")
+    if tn_count is None:
+        tn_count = out_tiles - tn_offset
+    if rows <= gemv_max_rows() and tn_offset == 0 and tn_count == out_tiles:
+        return inner_gem_fused(xh.reshape(rows, 1, n_in), trellis, k, cb)
+    if n_in % 64 or tn_count % 8 or tn_offset < 0 or tn_offset + tn_count > out_tiles:
+        raise ValueError("prefill GEMM needs in % 64 == 0 and a 128-column aligned slice")
+    y = torch.empty((rows, tn_count * 16), dtype=torch.float16, device=xh.device)
+    rc = _lib.load().exl3_gemm(
+        _ptr(xh), rows, n_in, _ptr(trellis), in_tiles, out_tiles, int(k), int(cb),
+        int(tn_offset), int(tn_count), _ptr(y), tn_count * 16, _stream(),
+    )
+    _lib.check(rc, "exl3_gemm")
+    return y
+
+
+def linear_forward(x2d, trellis, k, cb, suh=None, svh=None, bias=None, group_sub=None):
+    """Whole-layer forward on (rows, in) fp16 (``exl3_linear_forward``)."""
+    in_tiles, out_tiles = _trellis_dims(trellis, k)
+    _half(x2d, "x")
+    if x2d.dim() != 2 or x2d.shape[1] != in_tiles * 16:
+        raise ValueError(f"x must be (rows, {in_tiles * 16})")
+    rows = x2d.shape[0]
+    n_in, n_out = in_tiles * 16, out_tiles * 16
+    if n_in % 128 or n_out % 128:
+        raise ValueError("in/out features must be multiples of 128 for the Hadamard transform")
+    n_sub = 1
+    if suh is not None:
+        _half(suh, "suh")
+        n_sub = suh.shape[0] if suh.dim() == 2 else 1
+        if suh.shape[-1] != n_in:
+            raise ValueError("suh length does not match in_features")
+    for name, v in (("svh", svh), ("bias", bias)):
+        if v is not None:
+            _half(v, name)
+            if v.numel() != n_out:
+                raise ValueError(f"{name} length does not match out_features")
+    if group_sub is not None:
+        _check_cuda(group_sub, "group_sub")
+        if group_sub.dtype != torch.int32 or group_sub.numel() != n_out // 128:
+            raise ValueError("group_sub must be int32 with out_features/128 entries")
+    elif n_sub > 1:
+        raise ValueError("group_sub is required with stacked suh")
+    y = torch.empty((rows, n_out), dtype=torch.float16, device=x2d.device)
+    if rows == 0:
+        return y
+    lib = _lib.load()
+    ws_bytes = int(lib.exl3_linear_workspace_bytes(rows, n_in, n_out, n_sub))
+    ws = workspace(x2d.device, ws_bytes)
+    rc = lib.exl3_linear_forward(
+        _ptr(x2d), rows, _ptr(trellis), in_tiles, out_tiles, int(k), int(cb), _ptr(suh), n_sub,
+        _ptr(group_sub), _ptr(svh), _ptr(bias), _ptr(y), _ptr(ws), ws.numel(), _stream(),
+    )
+    _lib.check(rc, "exl3_linear_forward")
+    return y
+
+
+def moe_forward(x2d, indices, gu_trellis, gu_suh, gu_svh, dn_trellis, dn_suh, dn_svh, k, cb,
+                activation: int = 0):
+    """(T, D) fp16, (T, top_k) int32 -> (T, top_k, D) fp16 (``exl3_moe_forward``)."""
+    _half(x2d, "x")
+    _check_cuda(indices, "indices")
+    if indices.dtype != torch.int32 or indices.dim() != 2:
+        raise ValueError("indices must be int32 (tokens, top_k)")
+    T, D = x2d.shape
+    top_k = indices.shape[1]
+    E = gu_suh.shape[0]
+    H = dn_suh.shape[1]
+    y = torch.empty((T, top_k, D), dtype=torch.float16, device=x2d.device)
+    lib = _lib.load()
+    ws_bytes = int(lib.exl3_moe_workspace_bytes(T, top_k, D, H))
+    if ws_bytes == 0:
+        raise ValueError("MoE dims must be positive multiples of 128")
+    ws = workspace(x2d.device, ws_bytes)
+    rc = lib.exl3_moe_forward(
+        _ptr(x2d), T, _ptr(indices), top_k, _ptr(gu_trellis), _ptr(gu_suh), _ptr(gu_svh),
+        _ptr(dn_trellis), _ptr(dn_suh), _ptr(dn_svh), E, D, H, int(k), int(cb), int(activation),
+        _ptr(y), _ptr(ws), ws.numel(), _stream(),
+    )
+    _lib.check(rc, "exl3_moe_forward")
+    return y

@@ -1,0 +1,84 @@
+"""libexl3_hip.so loads without a GPU and exports exactly what include/exl3_hip.h
+declares; argument errors are reported as status codes before any launch."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from conftest import ROOT
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "exl3_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(exl3_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from ponyexl3_amd import _lib
+
+    assert os.path.exists(_lib.LIB_PATH), "build libexl3_hip.so first: python -m ponyexl3_amd.build"
+    return _lib.load()
+
+
+def test_every_declared_symbol_is_exported(lib):
+    names = _declared()
+    assert len(names) >= 12
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/exl3_hip.h but not exported"
+
+
+def test_binding_table_matches_header(lib):
+    from ponyexl3_amd import _lib
+
+    assert sorted(_lib.PROTOTYPES) == _declared()
+
+
+def test_version_and_status_strings(lib):
+    from ponyexl3_amd import _lib
+
+    assert lib.exl3_version() >= 100
+    assert _lib.status_string(0) == "ok"
+    for code in range(-8, 0):
+        assert _lib.status_string(code) not in ("", "unknown status")
+    assert lib.exl3_gemv_max_rows() == 8
+
+
+def test_argument_errors_before_launch(lib):
+    from ponyexl3_amd import _lib
+
+    p = ctypes.c_void_p(0x1000)  # never dereferenced: the checks below fail first
+    assert lib.exl3_decode_full(p, 1, 1, 9, 0, 0, 1, p, None) == _lib.EXL3_E_BAD_K
+    assert lib.exl3_decode_full(p, 1, 1, 4, 3, 0, 1, p, None) == _lib.EXL3_E_BAD_CODEBOOK
+    assert lib.exl3_decode_full(None, 1, 1, 4, 0, 0, 1, p, None) == _lib.EXL3_E_NULL_POINTER
+    assert lib.exl3_decode_full(p, 1, 1, 4, 0, 1, 1, p, None) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_had128_pre(p, 1, 100, None, 1, p, None) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_had128_post(p, 0, 2, 0, 1, 128, None, None, p, None) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_gemv(p, 9, 1, p, 8, 8, 4, 0, None, None, 1, p, p, 1 << 20, None) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_gemv(p, 1, 2, p, 8, 8, 4, 0, None, None, 1, p, p, 1 << 20, None) == _lib.EXL3_E_BAD_INDEX
+    assert lib.exl3_gemm(p, 32, 100, p, 8, 8, 4, 0, 0, 8, p, 128, None) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_linear_forward(p, 1, p, 8, 8, 4, 0, None, 1, None, None, None, p, p, 16, None) == _lib.EXL3_E_WORKSPACE
+    assert lib.exl3_linear_forward(p, 1, p, 7, 8, 4, 0, None, 1, None, None, None, p, p, 1 << 20, None) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_moe_forward(p, 1, p, 8, p, p, p, p, p, p, 4, 256, 100, 4, 0, 0, p, p, 1 << 20, None) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_moe_forward(p, 1, p, 8, p, p, p, p, p, p, 4, 256, 128, 4, 0, 7, p, p, 1 << 20, None) == _lib.EXL3_E_UNSUPPORTED
+
+
+def test_workspace_sizes(lib):
+    assert lib.exl3_gemv_workspace_bytes(1, 256, 32) >= 4096 * 4
+    assert lib.exl3_gemv_workspace_bytes(0, 256, 32) == 0
+    assert lib.exl3_linear_workspace_bytes(1, 4096, 4096, 1) > 4096 * 2
+    assert lib.exl3_linear_workspace_bytes(2048, 5120, 8192, 1) >= 2048 * (5120 + 8192) * 2
+    assert lib.exl3_moe_workspace_bytes(1, 8, 2048, 512) > 0
+    assert lib.exl3_moe_workspace_bytes(1, 8, 2048, 500) == 0
+
+
+def test_status_to_exception():
+    from ponyexl3_amd import _lib
+
+    _lib.check(0, "x")
+    with pytest.raises(ValueError):
+        _lib.check(_lib.EXL3_E_BAD_SHAPE, "x")
+    with pytest.raises(RuntimeError):
+        _lib.check(_lib.EXL3_E_LAUNCH, "x")
