@@ -97,6 +97,8 @@ def decode_full(trellis, k: int, cb: int, tn_offset: int = 0, tn_count: int | No
     if tn_offset < 0 or tn_count < 0 or tn_offset + tn_count > out_tiles:
         raise ValueError("slice exceeds output features")
     w = torch.empty((in_tiles * 16, tn_count * 16), dtype=torch.float16, device=trellis.device)
+    if w.numel() == 0:
+        return w
     rc = _lib.load().exl3_decode_full(
         _ptr(trellis), in_tiles, out_tiles, int(k), int(cb), int(tn_offset), int(tn_count),
         _ptr(w), _stream(),

@@ -1,0 +1,167 @@
+"""EXL3Linear / FusedEXL3Group against the oracle's layer forward
+(rel-L2 <= 1e-3, fp32 accumulation)."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import golden, rel_l2
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+def _x(rng, shape, device):
+    x = rng.standard_normal(shape).astype(np.float16)
+    return x, torch.from_numpy(x).to(device)
+
+
+def _oracle_forward(oracle, layer, x):
+    return oracle.linear_forward(layer.trellis, layer.k, layer.codebook_mode, layer.suh, layer.svh, x,
+                                 bias=layer.bias)
+
+
+def _golden_cases():
+    g = golden("forwards.npz")
+    return sorted({n[:-2] for n in g.files if n.endswith("_y")})
+
+
+@pytest.mark.parametrize("tag", _golden_cases())
+def test_golden_forward_outputs(cuda, tag):
+    """Outputs written by the reference's linear_forward_reconstruct."""
+    from ponyexl3_amd import EXL3Layer, EXL3Linear
+
+    g = golden("forwards.npz")
+    k = int(tag[1])
+    cb = int(tag.split("_")[1][2])
+    suh, svh = g[tag + "_suh"], g[tag + "_svh"]
+    if not tag.endswith("_bf"):
+        suh, svh = suh.view(np.float16), svh.view(np.float16)
+    bias = g[tag + "_bias"].view(np.float16) if tag + "_bias" in g.files else None
+    layer = EXL3Layer(tag, 128, 256, k, g[tag + "_trellis"], suh, svh, bias, mcg=cb == 1, mul1=cb == 2)
+    x = torch.from_numpy(g[tag + "_x"].view(np.float16)).to(cuda)
+    y = EXL3Linear(layer)(x).cpu().numpy()
+    assert rel_l2(y, g[tag + "_y"].view(np.float16)) <= TOL
+
+
+@pytest.mark.parametrize("rows", [1, 4, 8, 16, 19, 300])
+@pytest.mark.parametrize("k,mcg", [(2, True), (4, True), (4, False), (6, False)])
+def test_module_matches_oracle(cuda, oracle, rows, k, mcg):
+    from ponyexl3_amd import EXL3Linear, make_exl3_layer
+
+    layer = make_exl3_layer(k=k, in_features=256, out_features=384, seed=11 + k, mcg=mcg, bias=True)
+    rng = np.random.default_rng(rows)
+    x, xt = _x(rng, (rows, 256), cuda)
+    print(f"linear rows={rows} k={k} mcg={mcg}", flush=True)
+    y = EXL3Linear(layer)(xt).cpu().numpy()
+    assert y.dtype == np.float16 and y.shape == (rows, 384)
+    assert rel_l2(y, _oracle_forward(oracle, layer, x)) <= TOL
+
+
+def test_general_scales_not_only_signs(cuda, oracle):
+    from ponyexl3_amd import EXL3Linear, make_exl3_layer
+
+    rng = np.random.default_rng(21)
+    suh = (np.where(rng.random(256) > 0.5, -1, 1) * rng.uniform(0.25, 1.5, 256)).astype(np.float16)
+    svh = (np.where(rng.random(128) > 0.5, -1, 1) * rng.uniform(0.0, 2.0, 128)).astype(np.float16)
+    svh[:5] = 0  # dead columns
+    layer = make_exl3_layer(k=4, in_features=256, out_features=128, seed=3, suh=suh, svh=svh, mcg=True)
+    x, xt = _x(rng, (2, 256), cuda)
+    y = EXL3Linear(layer)(xt).cpu().numpy()
+    assert rel_l2(y, _oracle_forward(oracle, layer, x)) <= TOL
+    assert (y[:, :5] == 0).all()
+
+
+def test_module_keeps_leading_shape_and_has_no_parameters(cuda):
+    from ponyexl3_amd import EXL3Linear, make_exl3_layer
+
+    mod = EXL3Linear(make_exl3_layer(k=4, in_features=128, out_features=128, seed=3))
+    x = torch.zeros((2, 3, 128), dtype=torch.float16, device=cuda)
+    assert tuple(mod(x).shape) == (2, 3, 128)
+    assert list(mod.parameters()) == [] and list(mod.buffers()) == []
+    assert mod.state_dict() == {}
+    assert mod.in_features == 128 and mod.out_features == 128
+    mod.warm().release_source()
+    assert tuple(mod(x).shape) == (2, 3, 128)
+    with pytest.raises(ValueError):
+        mod(torch.zeros((1, 64), dtype=torch.float16, device=cuda))
+
+
+def test_config1_layer(cuda, oracle):
+    """4096 -> 4096, K=4, 3INST, x [1, 4096] ~ N(0, 1)."""
+    from ponyexl3_amd import EXL3Linear, make_exl3_layer
+
+    layer = make_exl3_layer(k=4, in_features=4096, out_features=4096, seed=10_004)
+    rng = np.random.default_rng(1)
+    x, xt = _x(rng, (1, 4096), cuda)
+    y = EXL3Linear(layer)(xt).cpu().numpy()
+    assert rel_l2(y, _oracle_forward(oracle, layer, x)) <= TOL
+
+
+@pytest.mark.parametrize("name,n_in,n_out", [("q_proj", 5120, 8192), ("k_proj", 5120, 1024),
+                                             ("o_proj", 8192, 5120), ("down_proj", 17408, 5120)])
+def test_config2_shapes_bs1(cuda, oracle, name, n_in, n_out):
+    from ponyexl3_amd import EXL3Linear, make_exl3_layer
+
+    layer = make_exl3_layer(k=4, in_features=n_in, out_features=n_out, seed=20_004)
+    rng = np.random.default_rng(2)
+    x, xt = _x(rng, (1, n_in), cuda)
+    print(f"config2 {name}", flush=True)
+    y = EXL3Linear(layer)(xt).cpu().numpy()
+    ref = oracle.linear_forward_bs1(layer.trellis, 4, 0, layer.suh, layer.svh, x[0])
+    assert rel_l2(y[0], ref) <= TOL
+
+
+@pytest.mark.parametrize("rows", [1, 8, 19])
+def test_fused_group_matches_members(cuda, oracle, rows):
+    from ponyexl3_amd import EXL3Linear, FusedEXL3Group, make_exl3_layer
+
+    layers = [make_exl3_layer(k=4, in_features=256, out_features=o, seed=70 + i, mcg=True, key=f"f{i}")
+              for i, o in enumerate((384, 256, 128))]
+    group = FusedEXL3Group(layers)
+    rng = np.random.default_rng(rows)
+    x, xt = _x(rng, (rows, 256), cuda)
+    outs = group.forward_all(xt)
+    for o, l in zip(outs, layers):
+        assert tuple(o.shape) == (rows, l.out_features)
+        assert rel_l2(o.cpu().numpy(), _oracle_forward(oracle, l, x)) <= TOL
+        member = EXL3Linear(l)(xt)  # tests/test_exl3_fused.py:32-48: max-rel < 5e-3
+        got, ref = o.float().cpu().numpy(), member.float().cpu().numpy()
+        assert np.abs(got - ref).max() / (np.abs(ref).max() + 1e-9) < 5e-3
+
+
+def test_fused_gate_up_config2(cuda, oracle):
+    """gate/up 5120 -> 17408 sibling-fused at batch 1."""
+    from ponyexl3_amd import FusedEXL3Group, make_exl3_layer
+
+    gate = make_exl3_layer(k=4, in_features=5120, out_features=17408, seed=20_104, key="gate")
+    up = make_exl3_layer(k=4, in_features=5120, out_features=17408, seed=20_204, key="up")
+    group = FusedEXL3Group([gate, up])
+    rng = np.random.default_rng(3)
+    x, xt = _x(rng, (1, 5120), cuda)
+    g_out, u_out = group.forward_all(xt)
+    for o, l in ((g_out, gate), (u_out, up)):
+        ref = oracle.linear_forward_bs1(l.trellis, 4, 0, l.suh, l.svh, x[0])
+        assert rel_l2(o.cpu().numpy()[0], ref) <= TOL
+
+
+def test_single_slot_cache_computes_once(cuda):
+    from ponyexl3_amd import FusedEXL3Group, make_exl3_layer
+
+    layers = [make_exl3_layer(k=4, in_features=256, out_features=128, seed=80 + i, key=f"c{i}") for i in range(2)]
+    group = FusedEXL3Group(layers)
+    s0, s1 = group.sibling(0), group.sibling(1)
+    calls = {"n": 0}
+    orig = group.forward_all
+
+    def counting(x):
+        calls["n"] += 1
+        return orig(x)
+
+    group.forward_all = counting
+    x = torch.zeros((1, 256), dtype=torch.float16, device=cuda)
+    s0(x)
+    s1(x)
+    assert calls["n"] == 1
+    s0(torch.zeros((1, 256), dtype=torch.float16, device=cuda))
+    assert calls["n"] == 2
+    assert s0.out_features == 128 and s0.in_features == 256

@@ -1,0 +1,129 @@
+"""Routed MoE expert chain against the oracle's unfused per-expert chain."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import rel_l2
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+def _experts(E, D, H, k, mcg, seed):
+    from ponyexl3_amd import make_exl3_layer
+
+    mk = lambda i, n_in, n_out, tag: make_exl3_layer(k=k, in_features=n_in, out_features=n_out,
+                                                     seed=seed + i, mcg=mcg, key=f"e{i}.{tag}")
+    gate = [mk(3 * e, D, H, "gate") for e in range(E)]
+    up = [mk(3 * e + 1, D, H, "up") for e in range(E)]
+    down = [mk(3 * e + 2, H, D, "down") for e in range(E)]
+    return gate, up, down
+
+
+def _oracle_chain(oracle, gate, up, down, x, idx, act):
+    experts = [{"gate": (g.trellis, g.suh, g.svh), "up": (u.trellis, u.suh, u.svh),
+                "down": (d.trellis, d.suh, d.svh)} for g, u, d in zip(gate, up, down)]
+    return oracle.moe_experts_forward(experts, x, idx, gate[0].k, gate[0].codebook_mode, act)
+
+
+@pytest.mark.parametrize("tokens", [1, 3, 8])
+@pytest.mark.parametrize("k,mcg,act", [(4, False, "silu"), (3, True, "silu"), (4, True, "gelu")])
+def test_moe_matches_oracle(cuda, oracle, tokens, k, mcg, act):
+    from ponyexl3_amd import EXL3SwitchGLU
+
+    E, D, H, kk = 6, 256, 128, 2
+    gate, up, down = _experts(E, D, H, k, mcg, 500)
+    moe = EXL3SwitchGLU.from_layers(gate, up, down, activation=act)
+    rng = np.random.default_rng(tokens + k)
+    x = (rng.standard_normal((tokens, D)) * 0.5).astype(np.float16)
+    idx = np.stack([rng.permutation(E)[:kk] for _ in range(tokens)]).astype(np.int32)
+    print(f"moe tokens={tokens} k={k} act={act}", flush=True)
+    y = moe(torch.from_numpy(x).to(cuda).reshape(1, tokens, D),
+            torch.from_numpy(idx).to(cuda).reshape(1, tokens, kk)).cpu().numpy()
+    assert y.shape == (1, tokens, kk, D)
+    ref = _oracle_chain(oracle, gate, up, down, x, idx, act)
+    assert rel_l2(y[0], ref) <= TOL
+
+
+def test_moe_equals_linear_modules(cuda):
+    """The stacked chain equals the same experts run as individual EXL3Linear
+    modules (fused-vs-unfused, ponyexl3/tests/test_moe_activation.py:44-65)."""
+    from ponyexl3_amd import EXL3Linear, EXL3SwitchGLU
+
+    E, D, H, kk = 4, 512, 256, 3
+    gate, up, down = _experts(E, D, H, 4, False, 900)
+    moe = EXL3SwitchGLU.from_layers(gate, up, down)
+    g = torch.Generator().manual_seed(1)
+    x = (torch.randn((2, D), generator=g) * 0.5).to(torch.float16).to(cuda)
+    idx = torch.tensor([[0, 2, 3], [1, 0, 2]], dtype=torch.int32, device=cuda)
+    y = moe(x.reshape(1, 2, D), idx.reshape(1, 2, kk))[0]
+    for t in range(2):
+        for s in range(kk):
+            e = int(idx[t, s])
+            gv = EXL3Linear(gate[e])(x[t : t + 1]).float()
+            uv = EXL3Linear(up[e])(x[t : t + 1]).float()
+            h = (torch.nn.functional.silu(gv) * uv).to(torch.float16)
+            ref = EXL3Linear(down[e])(h).float()
+            got = y[t, s].float()
+            assert float((got - ref[0]).abs().max() / (ref.abs().max() + 1e-9)) < 5e-3
+
+
+def test_config4_a3b_shapes(cuda):
+    """hidden 2048, 256 experts of 2048->512 / 512->2048, top-8 routing from a
+    softmax over seeded router logits, at 1 and 8 tokens. The result is checked
+    against per-expert EXL3Linear chains of the same (oracle-checked) kernels on
+    a sample of slots, and permutation equivariance over the slot order."""
+    from ponyexl3_amd import EXL3Layer, EXL3Linear, EXL3SwitchGLU, ops
+    from ponyexl3_amd.moe import combine_experts, route_topk
+
+    E, D, H, kk, k = 256, 2048, 512, 8, 4
+    rng = np.random.default_rng(40_004)
+    gu = rng.integers(0, 65536, size=(D // 16, E * 2 * H // 16, 16 * k), dtype=np.uint16)
+    dn = rng.integers(0, 65536, size=(H // 16, E * D // 16, 16 * k), dtype=np.uint16)
+    sgn = lambda shape: np.where(rng.random(shape) > 0.5, -1.0, 1.0).astype(np.float16)
+    gu_suh, gu_svh, dn_suh, dn_svh = sgn((E, 2, D)), sgn((E, 2 * H)), sgn((E, H)), sgn((E, D))
+    dev = lambda a: torch.from_numpy(a).to(cuda)
+    moe = EXL3SwitchGLU(gu_trellis=ops.as_trellis_tensor(gu, cuda), gu_suh=dev(gu_suh), gu_svh=dev(gu_svh),
+                        dn_trellis=ops.as_trellis_tensor(dn, cuda), dn_suh=dev(dn_suh), dn_svh=dev(dn_svh),
+                        k=k, cb=0)
+    for T in (1, 8):
+        x = (rng.standard_normal((T, D)) * 0.25).astype(np.float16)
+        logits = torch.from_numpy(rng.standard_normal((T, E)).astype(np.float32)).to(cuda)
+        inds, scores = route_topk(logits, kk)
+        assert torch.allclose(scores.sum(-1), torch.ones(T, device=cuda), atol=1e-5)
+        xt = dev(x)
+        print(f"config4 T={T}", flush=True)
+        y = moe(xt.reshape(1, T, D), inds.reshape(1, T, kk))
+        assert tuple(y.shape) == (1, T, kk, D)
+        out = combine_experts(y, scores.reshape(1, T, kk))
+        assert tuple(out.shape) == (1, T, D) and torch.isfinite(out.float()).all()
+        # slot-order permutation equivariance
+        perm = torch.randperm(kk, generator=torch.Generator().manual_seed(T)).to(cuda)
+        y2 = moe(xt.reshape(1, T, D), inds[:, perm].reshape(1, T, kk))
+        assert torch.equal(y2, y[:, :, perm])
+        # two sampled slots against stand-alone layers cut out of the stacks
+        gt = H // 16
+        for (t, s) in [(0, 0), (T - 1, kk - 1)]:
+            e = int(inds[t, s])
+            mk = lambda tr, suh, svh, n_in, n_out: EXL3Linear(
+                EXL3Layer(f"e{e}", n_in, n_out, k, np.ascontiguousarray(tr), suh, svh))
+            gl = mk(gu[:, e * gt : (e + 1) * gt], gu_suh[e, 0], gu_svh[e, :H], D, H)
+            ul = mk(gu[:, (E + e) * gt : (E + e + 1) * gt], gu_suh[e, 1], gu_svh[e, H:], D, H)
+            dl = mk(dn[:, e * (D // 16) : (e + 1) * (D // 16)], dn_suh[e], dn_svh[e], H, D)
+            h = (torch.nn.functional.silu(gl(xt[t : t + 1]).float()) * ul(xt[t : t + 1]).float()).to(torch.float16)
+            ref = dl(h).float()[0]
+            got = y[0, t, s].float()
+            assert float((got - ref).norm() / ref.norm()) <= 5e-3
+
+
+def test_errors(cuda):
+    from ponyexl3_amd import EXL3SwitchGLU
+
+    z = lambda *s: torch.zeros(s, dtype=torch.float16, device=cuda)
+    zi = lambda *s: torch.zeros(s, dtype=torch.int16, device=cuda)
+    with pytest.raises(ValueError):
+        EXL3SwitchGLU(gu_trellis=zi(8, 16, 64), gu_suh=z(1, 2, 128), gu_svh=z(1, 256), dn_trellis=zi(8, 8, 64),
+                      dn_suh=z(1, 128), dn_svh=z(1, 128), k=4, cb=0, activation="relu")
+    with pytest.raises(ValueError):
+        EXL3SwitchGLU(gu_trellis=zi(8, 8, 64), gu_suh=z(1, 2, 128), gu_svh=z(1, 256), dn_trellis=zi(8, 8, 64),
+                      dn_suh=z(1, 128), dn_svh=z(1, 128), k=4, cb=0)
