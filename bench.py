@@ -1,0 +1,347 @@
+#!/usr/bin/env python3
+"""Benchmark of the EXL3 quantized-linear hot path on one MI355X.
+
+A step is one pass over the linears of one 27B-class decoder layer at batch 1
+(q 5120->8192, k and v 5120->1024, o 8192->5120, gate+up 5120->17408 sibling
+fused, down 17408->5120; K=4, 3INST; seeded random trellis words, +-1 signs,
+fp16 x ~ N(0,1)): 180.9 MB of packed weights. Successive steps rotate over
+several distinct copies of the layer so the weights come from HBM, not from the
+256 MB last-level cache. ``value`` is effective weight bytes per second over the
+whole step (Hadamard kernels and launch gaps included).
+
+Prints ONE JSON line (see README / DESIGN.md for the fields). Extra objects:
+roofline (dominant kernel = the decode GEMV, timed per launch with HIP events),
+cpu_baseline (the C oracle on the host cores), prefill_gemm (M=2048, config 3)
+and moe (config 4).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+K_BITS = 4
+CB = 0
+
+# (name, in, out, members) of the config-2 layer; members > 1 = sibling-fused
+LAYER = [
+    ("q_proj", 5120, 8192, 1),
+    ("k_proj", 5120, 1024, 1),
+    ("v_proj", 5120, 1024, 1),
+    ("o_proj", 8192, 5120, 1),
+    ("gate_up", 5120, 17408, 2),
+    ("down_proj", 17408, 5120, 1),
+]
+
+
+def weight_bytes(n_in, n_out, members, k=K_BITS):
+    return n_in * n_out * members * k // 8
+
+
+def make_linear_np(n_in, n_out, members, seed, k=K_BITS):
+    """Seeded synthetic linear: raw random trellis words, +-1 signs (numpy)."""
+    rng = np.random.default_rng(seed)
+    trellis = rng.integers(0, 65536, size=(n_in // 16, n_out * members // 16, 16 * k), dtype=np.uint16)
+    suh = np.where(rng.random((members, n_in)) > 0.5, -1.0, 1.0).astype(np.float16)
+    svh = np.where(rng.random(n_out * members) > 0.5, -1.0, 1.0).astype(np.float16)
+    return trellis, suh, svh
+
+
+class DeviceLinear:
+    def __init__(self, name, n_in, n_out, members, seed, device):
+        import torch
+
+        from ponyexl3_amd import ops
+
+        tr, suh, svh = make_linear_np(n_in, n_out, members, seed)
+        self.name, self.n_in, self.n_out, self.members = name, n_in, n_out * members, members
+        self.trellis = ops.as_trellis_tensor(tr, device)
+        self.suh = torch.from_numpy(suh if members > 1 else suh[0]).to(device)
+        self.svh = torch.from_numpy(svh).to(device)
+        self.group_sub = None
+        if members > 1:
+            gs = np.repeat(np.arange(members, dtype=np.int32), n_out // 128)
+            self.group_sub = torch.from_numpy(gs).to(device)
+        self.bytes = weight_bytes(n_in, n_out, members)
+
+    def forward(self, x):
+        from ponyexl3_amd import ops
+
+        return ops.linear_forward(x, self.trellis, K_BITS, CB, self.suh, self.svh, None, self.group_sub)
+
+
+def cpu_baseline(budget_s=20.0):
+    """The C oracle (decode + Hadamard-128 + matvec, ponyexl3.ref restated) on
+    this host's cores over one config-2 layer; returns the JSON object."""
+    from oracle import exl3_oracle as orc
+
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
+    orc.set_num_threads(threads)
+    layers = []
+    for i, (name, n_in, n_out, members) in enumerate(LAYER):
+        tr, suh, svh = make_linear_np(n_in, n_out, members, 20_000 + 100 * i + K_BITS)
+        layers.append((tr, suh, svh, n_in, n_out, members))
+    x = {n: np.random.default_rng(n).standard_normal(n).astype(np.float16) for n in (5120, 8192, 17408)}
+    total = sum(weight_bytes(n_in, n_out, m) for _, n_in, n_out, m in LAYER)
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        for tr, suh, svh, n_in, n_out, members in layers:
+            for m in range(members):
+                cols = slice(m * n_out // 16, (m + 1) * n_out // 16)
+                orc.linear_forward_bs1(np.ascontiguousarray(tr[:, cols]), K_BITS, CB, suh[m],
+                                       svh[m * n_out : (m + 1) * n_out], x[n_in])
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt > budget_s or reps >= 50:
+            break
+    return {
+        "value": round(total * reps / dt / 1e9, 4),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"{reps} pass(es) over one config-2 decoder layer at batch 1 "
+                  f"({total / 1e6:.1f} MB of K=4 trellis, decode + Hadamard-128 + matvec), "
+                  f"C oracle with OpenMP, {dt:.1f} s",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--layers", type=int, default=4, help="distinct weight copies rotated over")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
+    ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--skip-extras", action="store_true", help="skip prefill GEMM and MoE figures")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build uses no second GPU, collectives or sharding; "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from ponyexl3_amd import _lib, ops
+
+    assert torch.cuda.is_available(), "no HIP device visible"
+    _lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    n_layers = max(1, args.layers)
+    layers = [
+        [DeviceLinear(n, i_, o_, m, 20_000 + 1000 * L + 100 * j + K_BITS, dev)
+         for j, (n, i_, o_, m) in enumerate(LAYER)]
+        for L in range(n_layers)
+    ]
+    bytes_per_step = sum(l.bytes for l in layers[0])
+    g = torch.Generator().manual_seed(1234)
+    xs = {n: torch.randn((1, n), generator=g).to(torch.float16).to(dev) for n in (5120, 8192, 17408)}
+
+    def step(L):
+        outs = []
+        for lin in layers[L]:
+            outs.append(lin.forward(xs[lin.n_in]))
+        return outs
+
+    for L in range(n_layers):  # grows the workspace, loads code objects
+        step(L)
+    torch.cuda.synchronize()
+
+    graphs = None
+    if not args.no_graph:
+        try:
+            graphs = []
+            for L in range(n_layers):
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr):
+                    keep = step(L)
+                graphs.append((gr, keep))
+            torch.cuda.synchronize()
+        except Exception as e:  # noqa: BLE001
+            print(f"HIP graph capture failed ({e!r}); timing eager launches", file=sys.stderr)
+            graphs = None
+
+    def run(i):
+        if graphs is not None:
+            graphs[i % n_layers][0].replay()
+        else:
+            step(i % n_layers)
+
+    for i in range(args.warmup):
+        run(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        run(i)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
+
+    # ---- roofline of the dominant kernel: the decode GEMV alone, per launch
+    per_linear = {}
+    reps = max(50, min(200, args.steps))
+    tot_bytes = tot_ms = 0.0
+    # 1 GiB streamed between timed launches pushes the previous weights out of
+    # the 256 MB last-level cache (the same linear of 4 layer copies would fit)
+    flush = torch.zeros(1 << 30, dtype=torch.int8, device=dev)
+    for j, (name, n_in, n_out, members) in enumerate(LAYER):
+        lins = [layers[L][j] for L in range(n_layers)]
+        xh = ops.had128_pre(xs[n_in], lins[0].suh).reshape(1, members, n_in).contiguous()
+        n_splits, _ = ops.gemv_plan(1, n_in // 16, lins[0].n_out // 128)
+        buf = torch.empty((n_splits, 1, lins[0].n_out), dtype=torch.float32, device=dev)
+        for r in range(10):
+            ops.inner_gemv_partials(xh, lins[r % n_layers].trellis, K_BITS, CB, lins[0].group_sub, out=buf)
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+        torch.cuda.synchronize()
+        for r in range(reps):
+            flush.add_(1)
+            evs[r][0].record()
+            ops.inner_gemv_partials(xh, lins[r % n_layers].trellis, K_BITS, CB, lins[0].group_sub, out=buf)
+            evs[r][1].record()
+        torch.cuda.synchronize()
+        ms = float(np.mean([a.elapsed_time(b) for a, b in evs]))
+        per_linear[name] = {"MB": round(lins[0].bytes / 1e6, 2), "us": round(ms * 1e3, 2),
+                            "GBps": round(lins[0].bytes / ms / 1e6, 1), "n_splits": n_splits}
+        tot_bytes += lins[0].bytes
+        tot_ms += ms
+    del flush
+    achieved = tot_bytes / tot_ms / 1e6
+    roofline = {
+        "bound": "hbm",
+        "kernel": "gemv_kernel<K=4, cb=3INST, rows=1>",
+        "achieved": round(achieved, 1),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4),
+        "traffic": None,
+        "bytes_per_launch": "in*out*K/8 of the launch's linear (sum over the 6 launches of a step / sum of their mean durations)",
+        "per_linear": per_linear,
+    }
+
+    extras = {}
+    if not args.skip_extras:
+        extras.update(bench_prefill(dev, layers[0], xs))
+        extras.update(bench_moe(dev))
+
+    out = {
+        "metric": "EXL3 GEMV effective GB/s (% HBM peak) at bs1; prefill GEMM TFLOPS at M=2048",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16 weights decoded from K-bit trellis codes, f32 accumulate",
+        "data": "synthetic (seeded random trellis words, +-1 signs, N(0,1) fp16 activations)",
+        "config": {
+            "workload": "configs[1]: 27B-class dense decoder linears at batch 1, K=4, 3INST; "
+                        "one step = q,k,v,o,gate+up(fused),down of one layer",
+            "bytes_per_step": bytes_per_step,
+            "weight_copies_rotated": n_layers,
+            "launch": "hip-graph replay" if graphs is not None else "eager",
+        },
+        "roofline": roofline,
+    }
+    out.update(extras)
+    if not args.skip_cpu:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+def _time_ms(fn, reps, warm=3):
+    import torch
+
+    for _ in range(warm):
+        fn()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    torch.cuda.synchronize()
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return float(np.mean([a.elapsed_time(b) for a, b in evs]))
+
+
+def bench_prefill(dev, layer, xs):
+    """config 3: M=2048 prefill GEMM on the config-2 weights (MFMA kernel alone)."""
+    import torch
+
+    from ponyexl3_amd import ops
+
+    g = torch.Generator().manual_seed(77)
+    per = {}
+    flop = ms_tot = 0.0
+    for lin in layer:
+        xh = torch.randn((2048, lin.n_in), generator=g).to(torch.float16).to(dev)
+        ms = _time_ms(lambda: ops.inner_gemm(xh, lin.trellis, K_BITS, CB), reps=10)
+        f = 2.0 * 2048 * lin.n_in * lin.n_out
+        per[lin.name] = {"ms": round(ms, 4), "TFLOPs": round(f / ms / 1e9, 1)}
+        flop += f
+        ms_tot += ms
+        del xh
+    tf = flop / ms_tot / 1e9
+    return {"prefill_gemm": {"M": 2048, "TFLOPs": round(tf, 1), "peak": MFMA_F16_PEAK_TFLOPS,
+                             "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "bound": "mfma",
+                             "kernel": "gemm_kernel<K=4, cb=3INST>", "per_linear": per}}
+
+
+def bench_moe(dev):
+    """config 4: A3B-style routed experts, top-8 of 256, 1 and 8 tokens."""
+    import torch
+
+    from ponyexl3_amd import EXL3SwitchGLU, ops
+    from ponyexl3_amd.moe import route_topk
+
+    E, D, H, kk = 256, 2048, 512, 8
+    copies = 2  # 2 x 403 MB of expert weights: more than the last-level cache
+    rng = np.random.default_rng(40_004)
+    moes = []
+    for c in range(copies):
+        gen = torch.Generator(device=dev).manual_seed(40_004 + c)
+        rnd = lambda *s: torch.randint(-32768, 32768, s, dtype=torch.int16, device=dev, generator=gen)
+        sgn = lambda *s: (torch.randint(0, 2, s, device=dev, generator=gen) * 2 - 1).to(torch.float16)
+        moes.append(EXL3SwitchGLU(
+            gu_trellis=rnd(D // 16, E * 2 * H // 16, 16 * K_BITS), gu_suh=sgn(E, 2, D), gu_svh=sgn(E, 2 * H),
+            dn_trellis=rnd(H // 16, E * D // 16, 16 * K_BITS), dn_suh=sgn(E, H), dn_svh=sgn(E, D),
+            k=K_BITS, cb=CB))
+    res = {}
+    for T in (1, 8):
+        x = torch.from_numpy((rng.standard_normal((1, T, D)) * 0.25).astype(np.float16)).to(dev)
+        logits = torch.from_numpy(rng.standard_normal((T, E)).astype(np.float32)).to(dev)
+        inds, _ = route_topk(logits, kk)
+        distinct = int(torch.unique(inds).numel())
+        idx = inds.reshape(1, T, kk)
+        it = [0]
+
+        def fn():
+            moes[it[0] % copies](x, idx)
+            it[0] += 1
+
+        ms = _time_ms(fn, reps=50)
+        nbytes = distinct * 3 * D * H * K_BITS // 8
+        res[f"tokens_{T}"] = {"us": round(ms * 1e3, 2), "distinct_experts": distinct,
+                              "MB": round(nbytes / 1e6, 2), "GBps": round(nbytes / ms / 1e6, 1),
+                              "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    return {"moe": res}
+
+
+if __name__ == "__main__":
+    main()

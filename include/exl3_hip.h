@@ -116,6 +116,22 @@ int exl3_gemv(const uint16_t *xh, int rows, int n_sub, const uint16_t *trellis, 
 size_t exl3_gemv_workspace_bytes(int rows, int in_tiles, int n_groups);
 
 /*
+ * The split-K plan exl3_gemv uses for a shape, and the decode-GEMV kernel on
+ * its own: writes the per-split fp32 partial sums without reducing them, the
+ * form the reference's launcher returns before its host-side sum
+ * ((n_splits, out) at ponyexl3/mlx/gemv_metal.py:1431-1457). The caller adds
+ * the slices in index order (exl3_had128_post does, fused with the output
+ * transform). One kernel launch, so it can be timed in isolation.
+ *   partial   fp32 [n_splits][rows][128*n_groups], n_splits from exl3_gemv_plan
+ */
+int exl3_gemv_plan(int rows, int in_tiles, int n_groups, int *n_splits, int *tile_rows_per_split);
+
+int exl3_gemv_partials(const uint16_t *xh, int rows, int n_sub, const uint16_t *trellis,
+                       int in_tiles, int out_tiles, int K, int cb, const int32_t *group_sub,
+                       const int32_t *group_tile, int n_groups, float *partial,
+                       size_t partial_bytes, void *stream);
+
+/*
  * Prefill GEMM: y = xh @ W_inner for rows > exl3_gemv_max_rows(), trellis tiles
  * decoded into LDS and contracted on fp16 MFMA with fp32 accumulation.
  * Replaces the rows > 16 branches of EXL3Linear.__call__

@@ -163,6 +163,30 @@ EXL3_EXPORT size_t exl3_gemv_workspace_bytes(int rows, int in_tiles, int n_group
     return (size_t)plan.n_splits * rows * n_groups * 128 * sizeof(float);
 }
 
+EXL3_EXPORT int exl3_gemv_plan(int rows, int in_tiles, int n_groups, int* n_splits,
+                               int* tile_rows_per_split) {
+    if (rows < 1 || rows > exl3::kGemvMaxRows || in_tiles < 1 || n_groups < 1)
+        return EXL3_E_BAD_SHAPE;
+    const exl3::GemvPlan plan = exl3::plan_gemv(rows, in_tiles, n_groups);
+    if (n_splits) *n_splits = plan.n_splits;
+    if (tile_rows_per_split) *tile_rows_per_split = plan.tk_per_split;
+    return EXL3_OK;
+}
+
+EXL3_EXPORT int exl3_gemv_partials(const uint16_t* xh, int rows, int n_sub, const uint16_t* trellis,
+                                   int in_tiles, int out_tiles, int K, int cb,
+                                   const int32_t* group_sub, const int32_t* group_tile,
+                                   int n_groups, float* partial, size_t partial_bytes,
+                                   void* stream) {
+    using namespace exl3;
+    if (rows < 1 || rows > kGemvMaxRows || in_tiles < 1 || n_groups < 1) return EXL3_E_BAD_SHAPE;
+    const GemvPlan plan = plan_gemv(rows, in_tiles, n_groups);
+    if (partial_bytes < (size_t)plan.n_splits * rows * n_groups * 128 * sizeof(float))
+        return EXL3_E_WORKSPACE;
+    return launch_gemv_partials(xh, rows, n_sub, trellis, in_tiles, out_tiles, K, cb, group_sub,
+                                group_tile, n_groups, partial, plan, as_stream(stream));
+}
+
 EXL3_EXPORT int exl3_gemv(const uint16_t* xh, int rows, int n_sub, const uint16_t* trellis,
                           int in_tiles, int out_tiles, int K, int cb, const int32_t* group_sub,
                           const int32_t* group_tile, int n_groups, float* y_out, void* workspace,

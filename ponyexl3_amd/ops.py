@@ -224,6 +224,41 @@ def inner_gem_fused(xh, trellis, k: int, cb: int, group_sub=None, group_tile=Non
     return y
 
 
+def gemv_plan(rows: int, in_tiles: int, n_groups: int) -> tuple[int, int]:
+    """(n_splits, tile rows per split) the small-batch kernel uses for a shape."""
+    a, b = ctypes.c_int(0), ctypes.c_int(0)
+    rc = _lib.load().exl3_gemv_plan(int(rows), int(in_tiles), int(n_groups), ctypes.byref(a),
+                                    ctypes.byref(b))
+    _lib.check(rc, "exl3_gemv_plan")
+    return a.value, b.value
+
+
+def inner_gemv_partials(xh, trellis, k: int, cb: int, group_sub=None, out=None):
+    """Decode-GEMV kernel alone: (n_splits, rows, out) fp32 partial sums
+    (``_run_inner_gem`` before its final sum, gemv_metal.py:1431-1457)."""
+    in_tiles, out_tiles = _trellis_dims(trellis, k)
+    _half(xh, "xh")
+    if xh.dim() != 3 or xh.shape[2] != in_tiles * 16:
+        raise ValueError("xh must be (rows, n_sub, in)")
+    rows, n_sub, _ = xh.shape
+    if (in_tiles * 16) % 128 or out_tiles % 8:
+        raise ValueError("in/out features must be multiples of 128")
+    if not 1 <= rows <= gemv_max_rows():
+        raise ValueError(f"rows must be in [1, {gemv_max_rows()}], got {rows}")
+    n_groups = out_tiles // 8
+    n_splits, _ = gemv_plan(rows, in_tiles, n_groups)
+    if out is None:
+        out = torch.empty((n_splits, rows, out_tiles * 16), dtype=torch.float32, device=xh.device)
+    elif out.dtype != torch.float32 or out.numel() < n_splits * rows * out_tiles * 16:
+        raise ValueError("out must be fp32 with n_splits*rows*out elements")
+    rc = _lib.load().exl3_gemv_partials(
+        _ptr(xh), rows, n_sub, _ptr(trellis), in_tiles, out_tiles, int(k), int(cb),
+        _ptr(group_sub), None, n_groups, _ptr(out), out.numel() * 4, _stream(),
+    )
+    _lib.check(rc, "exl3_gemv_partials")
+    return out
+
+
 def inner_gemv(xh, trellis, k: int, cb: int):
     """(in,) fp16 -> (out,) fp32 (``inner_gemv_mlx``, gemv_metal.py:1495-1505)."""
     if xh.dim() != 1:
