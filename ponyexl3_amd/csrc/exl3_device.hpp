@@ -61,29 +61,69 @@ enum : int { CB_3INST = 0, CB_MCG = 1, CB_MUL1 = 2 };
 // ponyexl3/ref/codebook.py:66-91.
 //
 // 3INST / MCG: x = cw*M + A (mod 2^32); x = (x & 0x8FFF8FFF) ^ 0x3B603B60; the
-// result is the fp16 sum of the two halves of x (one rounding). The 32-bit
-// product is built from two 16x16 multiplies (full rate) instead of one
-// v_mul_lo_u32 (quarter rate): cw*M = cw*Mlo + ((cw*Mhi) << 16) (mod 2^32).
+// result is the fp16 sum of the two halves of x (one rounding).
 //
 // MUL1: x = cw*0x83DCD12D; h = 1024 + (sum of the four bytes of x);
 // result = fp16(h * K_INV + K_BIAS). h*K_INV + K_BIAS is an integer multiple of
 // 2^-18 below 2^4, hence exact in fp32, so the single fp32->fp16 conversion is
 // the only rounding (the reference rounds once from double).
+//
+// Instruction choice follows measured gfx950 issue rates: v_mul_lo_u32 and
+// v_mad_u64_u32 run at the full 16 lanes/clk/SIMD, v_bitop3_b32 at the faster
+// rate of the simple ALU ops, and a v_add_f16 with SDWA operands adds the two
+// halves of one register and writes either half of the destination, so a pair
+// of weights is produced already packed for v_dot2_f32_f16 / MFMA.
+
+// x after the mask/xor step for 3INST and MCG.
 template <int CB>
-__device__ __forceinline__ half_t decode_cw(uint32_t cw) {
-    if constexpr (CB == CB_MUL1) {
-        const uint32_t x = cw * 0x83DCD12Du;
-        const uint32_t s = __builtin_amdgcn_sad_u8(x, 0u, 1024u);
-        const float v = __builtin_fmaf((float)s, 0.00676727294921875f, -10.3828125f);
-        return (half_t)v;
+__device__ __forceinline__ uint32_t scramble(uint32_t cw) {
+    static_assert(CB == CB_3INST || CB == CB_MCG, "MUL1 has its own path");
+    uint32_t x;
+    if constexpr (CB == CB_3INST) {
+        // one v_mad_u64_u32: the low dword of cw*M + A
+        uint64_t wide, carry;
+        const uint64_t addend = 64248484ull;
+        asm("v_mad_u64_u32 %0, %1, %2, %3, %4"
+            : "=v"(wide), "=s"(carry)
+            : "v"(cw), "s"(89226354u), "v"(addend));
+        x = (uint32_t)wide;
     } else {
-        constexpr uint32_t M = (CB == CB_3INST) ? 89226354u : 0xCBAC1FEDu;
-        constexpr uint32_t A = (CB == CB_3INST) ? 64248484u : 0u;
-        const uint32_t lo = cw * (M & 0xFFFFu) + A;
-        const uint32_t hi = cw * (M >> 16);
-        uint32_t x = lo + (hi << 16);
-        x = (x & 0x8FFF8FFFu) ^ 0x3B603B60u;
-        return bits_to_half((uint16_t)(x & 0xFFFFu)) + bits_to_half((uint16_t)(x >> 16));
+        x = cw * 0xCBAC1FEDu;
+    }
+    return __builtin_amdgcn_bitop3_b32(x, 0x8FFF8FFFu, 0x3B603B60u, 0x6A);  // c ^ (a & b)
+}
+
+// (half(x0.lo) + half(x0.hi), half(x1.lo) + half(x1.hi)) as a packed half2.
+__device__ __forceinline__ half2_t add_halves_pack(uint32_t x0, uint32_t x1) {
+    uint32_t r;
+    asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 "
+        "src1_sel:WORD_1"
+        : "=v"(r)
+        : "v"(x0));
+    asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 "
+        "src1_sel:WORD_1"
+        : "+v"(r)
+        : "v"(x1));
+    return bits_to_half2(r);
+}
+
+__device__ __forceinline__ half_t decode_mul1(uint32_t cw) {
+    const uint32_t x = cw * 0x83DCD12Du;
+    const uint32_t s = __builtin_amdgcn_sad_u8(x, 0u, 1024u);
+    const float v = __builtin_fmaf((float)s, 0.00676727294921875f, -10.3828125f);
+    return (half_t)v;
+}
+
+// Two codewords -> two packed fp16 weights.
+template <int CB>
+__device__ __forceinline__ half2_t decode_pair(uint32_t cw0, uint32_t cw1) {
+    if constexpr (CB == CB_MUL1) {
+        half2_t v;
+        v.x = decode_mul1(cw0);
+        v.y = decode_mul1(cw1);
+        return v;
+    } else {
+        return add_halves_pack(scramble<CB>(cw0), scramble<CB>(cw1));
     }
 }
 
@@ -147,10 +187,7 @@ __device__ __forceinline__ void decode_lane(const LaneWords<K>& lw, half2_t (&wp
         constexpr int n = 2 * pi.value;  // even codeword of the pair
         constexpr int cs = cw_col_sel(n);
         constexpr int j = cw_row(n) >> 1;  // x pair index
-        half2_t v;
-        v.x = decode_cw<CB>(lane_codeword<K, n>(lw));
-        v.y = decode_cw<CB>(lane_codeword<K, n + 1>(lw));
-        wp[8 * cs + j] = v;
+        wp[8 * cs + j] = decode_pair<CB>(lane_codeword<K, n>(lw), lane_codeword<K, n + 1>(lw));
     });
 }
 
