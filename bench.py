@@ -2,9 +2,12 @@
 """Benchmark of the EXL3 quantized-linear hot path on one MI355X.
 
 A step is one pass over the linears of one 27B-class decoder layer at batch 1
-(q 5120->8192, k and v 5120->1024, o 8192->5120, gate+up 5120->17408 sibling
-fused, down 17408->5120; K=4, 3INST; seeded random trellis words, +-1 signs,
-fp16 x ~ N(0,1)): 180.9 MB of packed weights. Successive steps rotate over
+(q 5120->8192 with k and v 5120->1024, o 8192->5120, gate+up 5120->17408,
+down 17408->5120; K=4, 3INST; seeded random trellis words, +-1 signs, fp16
+x ~ N(0,1)): 180.9 MB of packed weights. Linears that share an input run as one
+sibling-fused launch (gate+up, and q+k+v as the reference does for groups above
+64 MB of fp16-equivalent weights, ponyexl3/mlx/model.py:354-373), so a step is
+four launches; --unfused-qkv runs q, k and v as three. Successive steps rotate over
 several distinct copies of the layer so the weights come from HBM, not from the
 256 MB last-level cache. ``value`` is effective weight bytes per second over the
 whole step (Hadamard kernels and launch gaps included).
@@ -33,46 +36,52 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 K_BITS = 4
 CB = 0
 
-# (name, in, out, members) of the config-2 layer; members > 1 = sibling-fused
-LAYER = [
-    ("q_proj", 5120, 8192, 1),
-    ("k_proj", 5120, 1024, 1),
-    ("v_proj", 5120, 1024, 1),
-    ("o_proj", 8192, 5120, 1),
-    ("gate_up", 5120, 17408, 2),
-    ("down_proj", 17408, 5120, 1),
+# (name, in, [member out sizes]) of the config-2 layer; several members = sibling-fused
+LAYER_FUSED_QKV = [
+    ("qkv_proj", 5120, [8192, 1024, 1024]),
+    ("o_proj", 8192, [5120]),
+    ("gate_up", 5120, [17408, 17408]),
+    ("down_proj", 17408, [5120]),
 ]
+LAYER_SPLIT_QKV = [
+    ("q_proj", 5120, [8192]),
+    ("k_proj", 5120, [1024]),
+    ("v_proj", 5120, [1024]),
+] + LAYER_FUSED_QKV[1:]
+LAYER = LAYER_FUSED_QKV
 
 
-def weight_bytes(n_in, n_out, members, k=K_BITS):
-    return n_in * n_out * members * k // 8
+def weight_bytes(n_in, outs, k=K_BITS):
+    return n_in * sum(outs) * k // 8
 
 
-def make_linear_np(n_in, n_out, members, seed, k=K_BITS):
-    """Seeded synthetic linear: raw random trellis words, +-1 signs (numpy)."""
+def make_linear_np(n_in, outs, seed, k=K_BITS):
+    """Seeded synthetic linear(s): raw random trellis words, +-1 signs (numpy).
+    Members are concatenated along the tile columns, one suh row per member."""
     rng = np.random.default_rng(seed)
-    trellis = rng.integers(0, 65536, size=(n_in // 16, n_out * members // 16, 16 * k), dtype=np.uint16)
-    suh = np.where(rng.random((members, n_in)) > 0.5, -1.0, 1.0).astype(np.float16)
-    svh = np.where(rng.random(n_out * members) > 0.5, -1.0, 1.0).astype(np.float16)
+    trellis = rng.integers(0, 65536, size=(n_in // 16, sum(outs) // 16, 16 * k), dtype=np.uint16)
+    suh = np.where(rng.random((len(outs), n_in)) > 0.5, -1.0, 1.0).astype(np.float16)
+    svh = np.where(rng.random(sum(outs)) > 0.5, -1.0, 1.0).astype(np.float16)
     return trellis, suh, svh
 
 
 class DeviceLinear:
-    def __init__(self, name, n_in, n_out, members, seed, device):
+    def __init__(self, name, n_in, outs, seed, device):
         import torch
 
         from ponyexl3_amd import ops
 
-        tr, suh, svh = make_linear_np(n_in, n_out, members, seed)
-        self.name, self.n_in, self.n_out, self.members = name, n_in, n_out * members, members
+        tr, suh, svh = make_linear_np(n_in, outs, seed)
+        members = len(outs)
+        self.name, self.n_in, self.n_out, self.members = name, n_in, sum(outs), members
         self.trellis = ops.as_trellis_tensor(tr, device)
         self.suh = torch.from_numpy(suh if members > 1 else suh[0]).to(device)
         self.svh = torch.from_numpy(svh).to(device)
         self.group_sub = None
         if members > 1:
-            gs = np.repeat(np.arange(members, dtype=np.int32), n_out // 128)
+            gs = np.repeat(np.arange(members, dtype=np.int32), [o // 128 for o in outs])
             self.group_sub = torch.from_numpy(gs).to(device)
-        self.bytes = weight_bytes(n_in, n_out, members)
+        self.bytes = weight_bytes(n_in, outs)
 
     def forward(self, x):
         from ponyexl3_amd import ops
@@ -80,7 +89,7 @@ class DeviceLinear:
         return ops.linear_forward(x, self.trellis, K_BITS, CB, self.suh, self.svh, None, self.group_sub)
 
 
-def cpu_baseline(budget_s=20.0):
+def cpu_baseline(budget_s=12.0):
     """The C oracle (decode + Hadamard-128 + matvec, ponyexl3.ref restated) on
     this host's cores over one config-2 layer; returns the JSON object."""
     from oracle import exl3_oracle as orc
@@ -88,21 +97,22 @@ def cpu_baseline(budget_s=20.0):
     threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
     orc.set_num_threads(threads)
     layers = []
-    for i, (name, n_in, n_out, members) in enumerate(LAYER):
-        tr, suh, svh = make_linear_np(n_in, n_out, members, 20_000 + 100 * i + K_BITS)
-        layers.append((tr, suh, svh, n_in, n_out, members))
+    for i, (name, n_in, outs) in enumerate(LAYER):
+        tr, suh, svh = make_linear_np(n_in, outs, 20_000 + 100 * i + K_BITS)
+        c0 = 0
+        for m, n_out in enumerate(outs):  # the CPU runs the members one after the other
+            layers.append((np.ascontiguousarray(tr[:, c0 // 16 : (c0 + n_out) // 16]), suh[m],
+                           svh[c0 : c0 + n_out], n_in))
+            c0 += n_out
     x = {n: np.random.default_rng(n).standard_normal(n).astype(np.float16) for n in (5120, 8192, 17408)}
-    total = sum(weight_bytes(n_in, n_out, m) for _, n_in, n_out, m in LAYER)
+    total = sum(weight_bytes(n_in, outs) for _, n_in, outs in LAYER)
     reps, t0 = 0, time.perf_counter()
     while True:
-        for tr, suh, svh, n_in, n_out, members in layers:
-            for m in range(members):
-                cols = slice(m * n_out // 16, (m + 1) * n_out // 16)
-                orc.linear_forward_bs1(np.ascontiguousarray(tr[:, cols]), K_BITS, CB, suh[m],
-                                       svh[m * n_out : (m + 1) * n_out], x[n_in])
+        for tr, suh, svh, n_in in layers:
+            orc.linear_forward_bs1(tr, K_BITS, CB, suh, svh, x[n_in])
         reps += 1
         dt = time.perf_counter() - t0
-        if dt > budget_s or reps >= 50:
+        if dt > budget_s:
             break
     return {
         "value": round(total * reps / dt / 1e9, 4),
@@ -124,7 +134,11 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-extras", action="store_true", help="skip prefill GEMM and MoE figures")
+    ap.add_argument("--unfused-qkv", action="store_true", help="run q, k, v as three launches")
     args = ap.parse_args()
+    global LAYER
+    if args.unfused_qkv:
+        LAYER = LAYER_SPLIT_QKV
     if args.gpus != 1:
         print("bench.py measures one GPU: this build uses no second GPU, collectives or sharding; "
               "run with --gpus 1", file=sys.stderr)
@@ -141,8 +155,8 @@ def main():
 
     n_layers = max(1, args.layers)
     layers = [
-        [DeviceLinear(n, i_, o_, m, 20_000 + 1000 * L + 100 * j + K_BITS, dev)
-         for j, (n, i_, o_, m) in enumerate(LAYER)]
+        [DeviceLinear(n, i_, o_, 20_000 + 1000 * L + 100 * j + K_BITS, dev)
+         for j, (n, i_, o_) in enumerate(LAYER)]
         for L in range(n_layers)
     ]
     bytes_per_step = sum(l.bytes for l in layers[0])
@@ -197,9 +211,9 @@ def main():
     # 1 GiB streamed between timed launches pushes the previous weights out of
     # the 256 MB last-level cache (the same linear of 4 layer copies would fit)
     flush = torch.zeros(1 << 30, dtype=torch.int8, device=dev)
-    for j, (name, n_in, n_out, members) in enumerate(LAYER):
+    for j, (name, n_in, outs) in enumerate(LAYER):
         lins = [layers[L][j] for L in range(n_layers)]
-        xh = ops.had128_pre(xs[n_in], lins[0].suh).reshape(1, members, n_in).contiguous()
+        xh = ops.had128_pre(xs[n_in], lins[0].suh).reshape(1, len(outs), n_in).contiguous()
         n_splits, _ = ops.gemv_plan(1, n_in // 16, lins[0].n_out // 128)
         buf = torch.empty((n_splits, 1, lins[0].n_out), dtype=torch.float32, device=dev)
         for r in range(10):
@@ -227,7 +241,7 @@ def main():
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
         "traffic": None,
-        "bytes_per_launch": "in*out*K/8 of the launch's linear (sum over the 6 launches of a step / sum of their mean durations)",
+        "bytes_per_launch": "in*out*K/8 of the launch's linear(s): sum over the launches of a step / sum of their mean durations",
         "per_linear": per_linear,
     }
 
@@ -252,7 +266,7 @@ def main():
         "data": "synthetic (seeded random trellis words, +-1 signs, N(0,1) fp16 activations)",
         "config": {
             "workload": "configs[1]: 27B-class dense decoder linears at batch 1, K=4, 3INST; "
-                        "one step = q,k,v,o,gate+up(fused),down of one layer",
+                        "one step = " + ", ".join(n for n, _, _ in LAYER) + " of one layer",
             "bytes_per_step": bytes_per_step,
             "weight_copies_rotated": n_layers,
             "launch": "hip-graph replay" if graphs is not None else "eager",

@@ -156,11 +156,20 @@ int exl3_gemm(const uint16_t *xh, int rows, size_t ldx, const uint16_t *trellis,
  *   group_sub int32 [out/128] or NULL (required when n_sub > 1)
  *   y        fp16 [rows][out]
  *   workspace at least exl3_linear_workspace_bytes(rows, in, out, n_sub)
+ *   counters int32 [counters_len >= out/128] or NULL. With counters and
+ *            rows <= exl3_gemv_max_rows() the whole layer is ONE kernel launch:
+ *            the last wavefront to finish a 128-column group reduces the splits
+ *            and applies the output transform. The array must be all zero on
+ *            entry and is all zero again when the launch has finished, so a
+ *            caller zeroes it once and reuses it (calls that overlap on one
+ *            array race). NULL selects the three-launch chain
+ *            (exl3_had128_pre, exl3_gemv_partials, exl3_had128_post).
  */
 int exl3_linear_forward(const uint16_t *x, int rows, const uint16_t *trellis, int in_tiles,
                         int out_tiles, int K, int cb, const uint16_t *suh, int n_sub,
                         const int32_t *group_sub, const uint16_t *svh, const uint16_t *bias,
-                        uint16_t *y, void *workspace, size_t workspace_bytes, void *stream);
+                        uint16_t *y, void *workspace, size_t workspace_bytes, int32_t *counters,
+                        size_t counters_len, void *stream);
 
 size_t exl3_linear_workspace_bytes(int rows, int in_features, int out_features, int n_sub);
 

@@ -20,7 +20,7 @@ static LinearWorkspace linear_workspace(int rows, int in_features, int out_featu
     w.xh_bytes = align_up((size_t)rows * n_sub * in_features * 2, 256);
     if (rows <= kGemvMaxRows) {
         const GemvPlan plan = plan_gemv(rows, in_features / 16, out_features / 128);
-        w.second_bytes = (size_t)plan.n_splits * rows * out_features * sizeof(float);
+        w.second_bytes = (size_t)plan.n_partials() * rows * out_features * sizeof(float);
     } else {
         w.second_bytes = (size_t)rows * out_features * 2;
     }
@@ -57,7 +57,8 @@ EXL3_EXPORT int exl3_linear_forward(const uint16_t* x, int rows, const uint16_t*
                                     int in_tiles, int out_tiles, int K, int cb,
                                     const uint16_t* suh, int n_sub, const int32_t* group_sub,
                                     const uint16_t* svh, const uint16_t* bias, uint16_t* y,
-                                    void* workspace, size_t workspace_bytes, void* stream) {
+                                    void* workspace, size_t workspace_bytes, int32_t* counters,
+                                    size_t counters_len, void* stream) {
     using namespace exl3;
     if (int rc = check_k_cb(K, cb)) return rc;
     if (!x || !trellis || !y || !workspace) return EXL3_E_NULL_POINTER;
@@ -71,20 +72,26 @@ EXL3_EXPORT int exl3_linear_forward(const uint16_t* x, int rows, const uint16_t*
     uint16_t* xh = reinterpret_cast<uint16_t*>(workspace);
     char* second = reinterpret_cast<char*>(workspace) + ws.xh_bytes;
 
-    if (int rc = launch_had_pre(x, rows, in_features, suh, n_sub, xh, s)) return rc;
-
     if (rows <= kGemvMaxRows) {
         const int n_groups = out_tiles / 8;
         const GemvPlan plan = plan_gemv(rows, in_tiles, n_groups);
         float* partial = reinterpret_cast<float*>(second);
+        if (counters) {
+            // one launch: rotation, GEMV, split reduction and output transform fused
+            if (counters_len < (size_t)n_groups) return EXL3_E_WORKSPACE;
+            return launch_linear_small(x, rows, trellis, in_tiles, out_tiles, K, cb, suh, n_sub,
+                                       group_sub, svh, bias, y, partial, counters, plan, s);
+        }
+        if (int rc = launch_had_pre(x, rows, in_features, suh, n_sub, xh, s)) return rc;
         if (int rc = launch_gemv_partials(xh, rows, n_sub, trellis, in_tiles, out_tiles, K, cb,
                                           group_sub, nullptr, n_groups, partial, plan, s))
             return rc;
-        return launch_had_post(partial, 1, plan.n_splits, (size_t)rows * out_features, rows,
+        return launch_had_post(partial, 1, plan.n_partials(), (size_t)rows * out_features, rows,
                                out_features, svh, bias, y, s);
     }
 
-    // Prefill: one GEMM per run of 128-column groups that share an activation row.
+    // Prefill: rotation kernel, MFMA GEMM, output transform.
+    if (int rc = launch_had_pre(x, rows, in_features, suh, n_sub, xh, s)) return rc;
     uint16_t* ytmp = reinterpret_cast<uint16_t*>(second);
     if (n_sub == 1) {
         if (int rc = launch_gemm(xh, rows, (size_t)in_features, trellis, in_tiles, out_tiles, K, cb,

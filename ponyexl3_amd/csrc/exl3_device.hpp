@@ -167,14 +167,25 @@ __device__ __forceinline__ void load_lane_words(const uint32_t* __restrict__ bas
     for (int i = 0; i < K; i++) own[i] = p[i];
 }
 
-template <int K>
-__device__ __forceinline__ LaneWords<K> finish_lane_words(const uint32_t (&own)[K], int lane) {
-    LaneWords<K> lw;
+// The dword that precedes a lane's own K dwords: the last dword of lane u-1 of
+// the same tile (u = 0 wraps to u = 7, the stream is circular). One ds_bpermute.
+__device__ __forceinline__ uint32_t neighbour_word(uint32_t last_own, int lane) {
     const int src = (lane & ~7) | ((lane + 7) & 7);
-    lw.w[0] = (uint32_t)__shfl((int)own[K - 1], src, kWave);
+    return (uint32_t)__shfl((int)last_own, src, kWave);
+}
+
+template <int K>
+__device__ __forceinline__ LaneWords<K> make_lane_words(uint32_t prev, const uint32_t (&own)[K]) {
+    LaneWords<K> lw;
+    lw.w[0] = prev;
 #pragma unroll
     for (int i = 0; i < K; i++) lw.w[i + 1] = own[i];
     return lw;
+}
+
+template <int K>
+__device__ __forceinline__ LaneWords<K> finish_lane_words(const uint32_t (&own)[K], int lane) {
+    return make_lane_words<K>(neighbour_word(own[K - 1], lane), own);
 }
 
 // Decodes the lane's 32 codewords into 16 half2 pairs.

@@ -53,16 +53,26 @@ constexpr int kGemvMaxRows = 8;
 // into n_splits ranges of tk_per_split rows; every (128-column group, split)
 // pair is one workgroup.
 struct GemvPlan {
-    int n_splits;
-    int tk_per_split;
+    int n_splits;      // wave-level splits of the tile rows
+    int tk_per_split;  // tile rows per split
+    // the four waves of a workgroup are summed in LDS: partial rows per group
+    int n_partials() const { return (n_splits + 3) / 4; }
 };
 GemvPlan plan_gemv(int rows, int in_tiles, int n_groups);
 
-// partial: fp32 [n_splits][rows][128*n_groups]
+// partial: fp32 [plan.n_partials()][rows][128*n_groups]
 int launch_gemv_partials(const uint16_t* xh, int rows, int n_sub, const uint16_t* trellis,
                          int in_tiles, int out_tiles, int K, int cb, const int32_t* group_sub,
                          const int32_t* group_tile, int n_groups, float* partial, GemvPlan plan,
                          hipStream_t stream);
+
+// One-launch small-batch layer (rows <= kGemvMaxRows): counters[out_tiles/8] must
+// be zero on entry and are zero again on exit.
+int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, int in_tiles,
+                        int out_tiles, int K, int cb, const uint16_t* suh, int n_sub,
+                        const int32_t* group_sub, const uint16_t* svh, const uint16_t* bias,
+                        uint16_t* y, float* partial, int* counters, GemvPlan plan,
+                        hipStream_t stream);
 
 int launch_had_pre(const uint16_t* x, int rows, int n, const uint16_t* suh, int n_sub,
                    uint16_t* xh, hipStream_t stream);

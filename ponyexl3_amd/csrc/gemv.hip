@@ -5,7 +5,7 @@
 //   * the unit of work is a wavefront: wave (g, s) owns the 128-column output
 //     group g and split s of the tile rows, tk in [s*L, min(in_tiles, (s+1)*L));
 //     the four waves of a workgroup are four consecutive splits of one group and
-//     never talk to each other (no LDS, no barrier);
+//     meet only once, at the end, to add their accumulators through LDS;
 //   * per tile row a wave issues one wave-wide non-temporal load of 256*K
 //     contiguous bytes (8 tiles) and keeps kPrefetch such loads in flight; lane
 //     u of a tile decodes its 32 codewords = output columns u and u+8 over all 16
@@ -13,7 +13,7 @@
 //     cross-lane reduction exists anywhere;
 //   * activations of a tile row are wave-uniform (scalar loads) and enter
 //     v_dot2_f32_f16 as SGPR operands;
-//   * every wave writes one fp32 partial row [split][row][128 columns]; splits
+//   * every workgroup writes one fp32 partial row [wg][row][128 columns]; rows
 //     are added in index order by the caller (exl3_had128_post or the reduction
 //     kernel below) - no atomics, so results are run-to-run deterministic.
 //
@@ -30,7 +30,7 @@
 
 namespace exl3 {
 
-constexpr int kPrefetch = 4;  // wave-wide loads in flight per wave
+constexpr int kPrefetch = 6;  // wave-wide loads in flight per wave
 
 template <int K>
 __device__ __forceinline__ void load_lane_words_nt(const uint32_t* __restrict__ p,
@@ -49,12 +49,12 @@ __global__ __launch_bounds__(256) void gemv_kernel(
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int split = blockIdx.y * 4 + wave;
-    if (split >= n_splits) return;
+    const bool active = split < n_splits;  // idle waves still reach the barrier below
     const int tn0 = group_tile ? group_tile[g] : g * 8;
     const int sub = group_sub ? group_sub[g] : 0;
     const int in_features = in_tiles * 16;
-    const int tk_begin = split * tk_per_split;
-    const int tk_end = min(in_tiles, tk_begin + tk_per_split);
+    const int tk_begin = active ? split * tk_per_split : 0;
+    const int tk_end = active ? min(in_tiles, tk_begin + tk_per_split) : 0;
     const size_t row_words = (size_t)out_tiles * (8 * K);
     const uint32_t* base = trellis + (size_t)tn0 * (8 * K) + lane * K;
 
@@ -73,54 +73,342 @@ __global__ __launch_bounds__(256) void gemv_kernel(
     // is refilled only after its codewords have been consumed, so the refill can
     // land in the same registers and the only wait in the loop is for the oldest
     // of the kPrefetch loads in flight.
+    // One pipeline step: the neighbour dword and (for one or two batch rows) the
+    // activations of the NEXT tile row are requested first, so the LDS-crossbar
+    // and scalar-cache latencies hide behind this step's decode; then the current
+    // slot is decoded and multiplied, then the slot is refilled from memory.
+    constexpr bool kPipeX = MT <= 2;  // more rows would not fit the scalar registers
+    struct XTile {
+        half2_t v[MT][8];
+    };
+    auto load_x = [&](int tk) {
+        XTile t;
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            const half2_t* xp = reinterpret_cast<const half2_t*>(xrow[m] + tk * 16);
+#pragma unroll
+            for (int j = 0; j < 8; j++) t.v[m][j] = xp[j];
+        }
+        return t;
+    };
+    auto consume = [&](const uint32_t (&words)[K], uint32_t prev, const XTile& xt) {
+        const LaneWords<K> lw = make_lane_words<K>(prev, words);
+        half2_t wp[16];
+        decode_lane<K, CB>(lw, wp);
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                acc[m][0] = dot2(wp[j], xt.v[m][j], acc[m][0]);
+                acc[m][1] = dot2(wp[8 + j], xt.v[m][j], acc[m][1]);
+            }
+        }
+    };
+
+    if (active) {
+        uint32_t buf[kPrefetch][K];
+#pragma unroll
+        for (int s = 0; s < kPrefetch; s++) {
+            const int t = min(tk_begin + s, tk_end - 1);  // clamped: stays inside the split
+            load_lane_words_nt<K>(base + (size_t)t * row_words, buf[s]);
+        }
+        uint32_t prev = neighbour_word(buf[0][K - 1], lane);
+        XTile xcur = load_x(tk_begin);
+        int tk0 = tk_begin;
+        for (; tk0 + kPrefetch <= tk_end; tk0 += kPrefetch) {
+#pragma unroll
+            for (int s = 0; s < kPrefetch; s++) {
+                const int tk = tk0 + s;
+                // results requested one step ago (scalar loads return out of order, so
+                // the only usable wait is for all of them) - long since complete
+                __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+                __builtin_amdgcn_sched_barrier(0);
+                const uint32_t prev_next = neighbour_word(buf[(s + 1) % kPrefetch][K - 1], lane);
+                XTile xnext;
+                if constexpr (kPipeX) xnext = load_x(min(tk + 1, tk_end - 1));
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (!kPipeX) xcur = load_x(tk);
+                consume(buf[s], prev, xcur);
+                const int tn = min(tk + kPrefetch, tk_end - 1);
+                load_lane_words_nt<K>(base + (size_t)tn * row_words, buf[s]);
+                __builtin_amdgcn_sched_barrier(0);
+                prev = prev_next;
+                if constexpr (kPipeX) xcur = xnext;
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < kPrefetch - 1; s++) {
+            const int tk = tk0 + s;
+            if (tk < tk_end) {
+                const uint32_t prev_next = neighbour_word(buf[(s + 1) % kPrefetch][K - 1], lane);
+                xcur = load_x(tk);
+                consume(buf[s], prev, xcur);
+                prev = prev_next;
+            }
+        }
+    }
+
+    // the four waves are summed through LDS in wave order; one partial row per workgroup
+    __shared__ float red[4][MT][128];
+    const int c0 = (lane >> 3) * 16 + (lane & 7);
+#pragma unroll
+    for (int m = 0; m < MT; m++) {
+        red[wave][m][c0] = acc[m][0];
+        red[wave][m][c0 + 8] = acc[m][1];
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const size_t out_total = (size_t)n_groups * 128;
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            if (m < rows) {
+                float2_t v;
+                v.x = ((red[0][m][2 * lane] + red[1][m][2 * lane]) + red[2][m][2 * lane]) +
+                      red[3][m][2 * lane];
+                v.y = ((red[0][m][2 * lane + 1] + red[1][m][2 * lane + 1]) +
+                       red[2][m][2 * lane + 1]) + red[3][m][2 * lane + 1];
+                *reinterpret_cast<float2_t*>(partial + ((size_t)blockIdx.y * rows + m) * out_total +
+                                             (size_t)g * 128 + 2 * lane) = v;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Whole small-batch layer in one launch: input Hadamard, decode GEMV, split
+// reduction, output Hadamard, svh and bias.
+//
+//   * input side: a wave rotates the 128-wide block of x (times suh) that its
+//     current tile rows need, keeps the fp16 result in its own LDS slot and reads
+//     the 16 activations of a tile row back with two broadcast ds_read_b128; the
+//     raw block after that is already in flight while the current one is used;
+//   * output side: every wave stores its fp32 partial row, then bumps the
+//     counter of its 128-column group; the wave that brings the counter to
+//     n_splits adds the partials in split order, rounds to fp16 (the cast at
+//     ponyexl3/ref/forward.py:41), applies the output Hadamard of that one
+//     128-column block, svh and bias, and resets the counter to zero. No wave
+//     ever waits for another one, and the sum order is fixed, so the result is
+//     deterministic.
+// Counters must be zero on entry; they are zero again when the kernel ends.
+constexpr float kHadScaleF = 0.088388347648318440550f;  // 1/sqrt(128)
+
+__device__ __forceinline__ void wht128_lanes(float& a, float& b, int lane) {
+    const float s = a + b, d = a - b;
+    a = s;
+    b = d;
+#pragma unroll
+    for (int bit = 0; bit < 6; bit++) {
+        const int mask = 1 << bit;
+        const float pa = __shfl_xor(a, mask, kWave);
+        const float pb = __shfl_xor(b, mask, kWave);
+        const bool upper = (lane & mask) != 0;
+        a = upper ? pa - a : a + pa;
+        b = upper ? pb - b : b + pb;
+    }
+}
+
+template <int K, int CB, int MT>
+__global__ __launch_bounds__(256) void linear_small_kernel(
+    const uint32_t* __restrict__ trellis, const half_t* __restrict__ x,
+    const half_t* __restrict__ suh, const half_t* __restrict__ svh,
+    const half_t* __restrict__ bias, half_t* __restrict__ y, float* partial, int* counters,
+    const int* __restrict__ group_sub, int in_tiles, int out_tiles, int rows, int n_groups,
+    int tk_per_split, int n_splits) {
+    __shared__ __attribute__((aligned(16))) half_t xs[4][MT][128];
+    const int g = blockIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int split = blockIdx.y * 4 + wave;
+    const bool active = split < n_splits;  // idle waves still take part in the barriers below
+    const int sub = group_sub ? group_sub[g] : 0;
+    const int in_features = in_tiles * 16;
+    const int tk_begin = active ? split * tk_per_split : 0;
+    const int tk_end = active ? min(in_tiles, tk_begin + tk_per_split) : 0;
+    const size_t row_words = (size_t)out_tiles * (8 * K);
+    const uint32_t* base = trellis + (size_t)g * 8 * (8 * K) + lane * K;
+    const half_t* suh_row = suh ? suh + (size_t)sub * in_features : nullptr;
+
+    float acc[MT][2];
+#pragma unroll
+    for (int m = 0; m < MT; m++) acc[m][0] = acc[m][1] = 0.f;
+
+    // ---- input Hadamard, one 128-block (8 tile rows) at a time
+    half2_t xraw[MT], sraw;
+    auto fetch_block = [&](int blk) {
+        const int off = blk * 128 + 2 * lane;
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            const int r = m < rows ? m : 0;
+            xraw[m] = *reinterpret_cast<const half2_t*>(x + (size_t)r * in_features + off);
+        }
+        if (suh_row) sraw = *reinterpret_cast<const half2_t*>(suh_row + off);
+    };
+    auto rotate_block = [&]() {
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            float a = (float)xraw[m].x, b = (float)xraw[m].y;
+            if (suh_row) {
+                a = __fmul_rn(a, (float)sraw.x);
+                b = __fmul_rn(b, (float)sraw.y);
+            }
+            wht128_lanes(a, b, lane);
+            half2_t o;
+            o.x = (half_t)__fmul_rn(a, kHadScaleF);
+            o.y = (half_t)__fmul_rn(b, kHadScaleF);
+            *reinterpret_cast<half2_t*>(&xs[wave][m][2 * lane]) = o;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+
     auto consume = [&](const uint32_t (&words)[K], int tk) {
+        if ((tk & 7) == 0 && tk != tk_begin) {  // entering the next Hadamard block
+            rotate_block();
+            if (tk + 8 < tk_end) fetch_block((tk >> 3) + 1);
+        }
         const LaneWords<K> lw = finish_lane_words<K>(words, lane);
         half2_t wp[16];
         decode_lane<K, CB>(lw, wp);
 #pragma unroll
         for (int m = 0; m < MT; m++) {
-            const half2_t* xp = reinterpret_cast<const half2_t*>(xrow[m] + tk * 16);
+            const uint4_t* xp = reinterpret_cast<const uint4_t*>(&xs[wave][m][(tk & 7) * 16]);
+            const uint4_t x0 = xp[0], x1 = xp[1];
+            const half2_t xv[8] = {bits_to_half2(x0.x), bits_to_half2(x0.y), bits_to_half2(x0.z),
+                                   bits_to_half2(x0.w), bits_to_half2(x1.x), bits_to_half2(x1.y),
+                                   bits_to_half2(x1.z), bits_to_half2(x1.w)};
 #pragma unroll
             for (int j = 0; j < 8; j++) {
-                const half2_t xv = xp[j];
-                acc[m][0] = dot2(wp[j], xv, acc[m][0]);
-                acc[m][1] = dot2(wp[8 + j], xv, acc[m][1]);
+                acc[m][0] = dot2(wp[j], xv[j], acc[m][0]);
+                acc[m][1] = dot2(wp[8 + j], xv[j], acc[m][1]);
             }
         }
     };
 
-    uint32_t buf[kPrefetch][K];
-#pragma unroll
-    for (int s = 0; s < kPrefetch; s++) {
-        const int t = min(tk_begin + s, tk_end - 1);  // clamped: stays inside the split
-        load_lane_words_nt<K>(base + (size_t)t * row_words, buf[s]);
-    }
-    int tk0 = tk_begin;
-    for (; tk0 + kPrefetch <= tk_end; tk0 += kPrefetch) {
+    if (active) {
+        uint32_t buf[kPrefetch][K];
 #pragma unroll
         for (int s = 0; s < kPrefetch; s++) {
-            consume(buf[s], tk0 + s);
-            const int tn = min(tk0 + s + kPrefetch, tk_end - 1);
-            load_lane_words_nt<K>(base + (size_t)tn * row_words, buf[s]);
+            const int t = min(tk_begin + s, tk_end - 1);
+            load_lane_words_nt<K>(base + (size_t)t * row_words, buf[s]);
         }
-    }
-#pragma unroll
-    for (int s = 0; s < kPrefetch - 1; s++)
-        if (tk0 + s < tk_end) consume(buf[s], tk0 + s);
+        fetch_block(tk_begin >> 3);
+        rotate_block();
+        if (((tk_begin >> 3) + 1) * 8 < tk_end) fetch_block((tk_begin >> 3) + 1);
 
+        int tk0 = tk_begin;
+        for (; tk0 + kPrefetch <= tk_end; tk0 += kPrefetch) {
+#pragma unroll
+            for (int s = 0; s < kPrefetch; s++) {
+                consume(buf[s], tk0 + s);
+                const int tn = min(tk0 + s + kPrefetch, tk_end - 1);
+                load_lane_words_nt<K>(base + (size_t)tn * row_words, buf[s]);
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < kPrefetch - 1; s++)
+            if (tk0 + s < tk_end) consume(buf[s], tk0 + s);
+    }
+
+    // ---- the four waves of the workgroup are summed through LDS in wave order,
+    // the workgroup stores ONE fp32 partial row, and the last workgroup of the
+    // 128-column group finishes the columns.
+    // The eight XCDs have private L2 caches, so a device-scope release/acquire
+    // fence would write back / invalidate a whole L2 per workgroup. Instead the
+    // data that crosses workgroups (partials, counters) only ever moves through
+    // device-scope accesses, which bypass the non-coherent cache levels: the
+    // partial stores are waited for before the counter is bumped, and the
+    // finishing workgroup reads them back with device-scope loads.
+    __shared__ float red[4][MT][128];
+    __shared__ int last_flag;
     const int c0 = (lane >> 3) * 16 + (lane & 7);
-    const size_t out_total = (size_t)n_groups * 128;
 #pragma unroll
     for (int m = 0; m < MT; m++) {
-        if (m < rows) {
-            float* dst = partial + ((size_t)split * rows + m) * out_total + (size_t)g * 128 + c0;
-            dst[0] = acc[m][0];
-            dst[8] = acc[m][1];
+        red[wave][m][c0] = acc[m][0];
+        red[wave][m][c0 + 8] = acc[m][1];
+    }
+    __syncthreads();
+    const size_t out_total = (size_t)n_groups * 128;
+    const int wg_splits = (n_splits + 3) >> 2;  // partial rows per group
+    const size_t col = (size_t)g * 128 + 2 * lane;
+    if (wave == 0) {
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            if (m < rows) {
+                float2_t v;
+                v.x = ((red[0][m][2 * lane] + red[1][m][2 * lane]) + red[2][m][2 * lane]) +
+                      red[3][m][2 * lane];
+                v.y = ((red[0][m][2 * lane + 1] + red[1][m][2 * lane + 1]) +
+                       red[2][m][2 * lane + 1]) + red[3][m][2 * lane + 1];
+                uint64_t* dst = reinterpret_cast<uint64_t*>(
+                    partial + ((size_t)blockIdx.y * rows + m) * out_total + col);
+                __hip_atomic_store(dst, __builtin_bit_cast(uint64_t, v), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        int seen = 0;
+        if (lane == 0) {
+            seen = __hip_atomic_fetch_add(&counters[g], 1, __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT);
+            last_flag = seen == wg_splits - 1;
         }
     }
+    __syncthreads();
+    if (!last_flag) return;
+    asm volatile("" ::: "memory");
+    half2_t sv, bv;
+    if (svh) sv = *reinterpret_cast<const half2_t*>(svh + col);
+    if (bias) bv = *reinterpret_cast<const half2_t*>(bias + col);
+    for (int m = wave; m < rows; m += 4) {  // the finishing workgroup splits the batch rows
+        // device-scope loads, sixteen partial rows in flight, added in split order
+        const float* src = partial + (size_t)m * out_total + col;
+        const size_t stride = (size_t)rows * out_total;
+        float a = 0.f, b = 0.f;
+        int s = 0;
+        for (; s + 16 <= wg_splits; s += 16) {
+            uint64_t v[16];
+#pragma unroll
+            for (int i = 0; i < 16; i++)
+                v[i] = __hip_atomic_load(
+                    reinterpret_cast<const uint64_t*>(src + (size_t)(s + i) * stride),
+                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const float2_t f = __builtin_bit_cast(float2_t, v[i]);
+                a = __fadd_rn(a, f.x);
+                b = __fadd_rn(b, f.y);
+            }
+        }
+        for (; s < wg_splits; s++) {
+            const float2_t f = __builtin_bit_cast(
+                float2_t, __hip_atomic_load(reinterpret_cast<const uint64_t*>(src + (size_t)s * stride),
+                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            a = __fadd_rn(a, f.x);
+            b = __fadd_rn(b, f.y);
+        }
+        a = (float)(half_t)a;
+        b = (float)(half_t)b;
+        wht128_lanes(a, b, lane);
+        a = __fmul_rn(a, kHadScaleF);
+        b = __fmul_rn(b, kHadScaleF);
+        if (svh) {
+            a = __fmul_rn(a, (float)sv.x);
+            b = __fmul_rn(b, (float)sv.y);
+        }
+        half2_t o;
+        o.x = (half_t)a;
+        o.y = (half_t)b;
+        if (bias) {
+            o.x = o.x + bv.x;
+            o.y = o.y + bv.y;
+        }
+        *reinterpret_cast<half2_t*>(y + (size_t)m * out_total + col) = o;
+    }
+    if (threadIdx.x == 0)
+        __hip_atomic_store(&counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// y[i] = sum over splits, index order.
+// y[i] = sum over the partial rows, index order.
 __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ partial,
                                                               float* __restrict__ y, size_t n,
                                                               int n_splits) {
@@ -142,10 +430,11 @@ static int env_int(const char* name, int dflt, int lo, int hi) {
 
 GemvPlan plan_gemv(int rows, int in_tiles, int n_groups) {
     (void)rows;
-    // All waves of a launch should be resident together and carry equal work:
-    // aim for kWavesPerSimd waves on each of the 256*4 SIMDs, but never fewer
+    // Aim for kWavesPerSimd waves per SIMD over the 256*4 SIMDs, but never fewer
     // than kMinTileRows tile rows per wave (pipeline depth, partial-sum traffic).
-    static const int kWavesPerSimd = env_int("EXL3_GEMV_WAVES_PER_SIMD", 4, 1, 16);
+    // Measured on gate+up (272 groups): 4 waves/SIMD leaves workgroup counts like
+    // 4.25 per CU, and the CUs that draw 5 set the kernel time; 12 dilutes that.
+    static const int kWavesPerSimd = env_int("EXL3_GEMV_WAVES_PER_SIMD", 12, 1, 16);
     static const int kMinTileRows = env_int("EXL3_GEMV_MIN_TILE_ROWS", 8, 1, 4096);
     const int target_waves = 256 * 4 * kWavesPerSimd;
     int n_splits = target_waves / (n_groups > 0 ? n_groups : 1);
@@ -190,6 +479,42 @@ int launch_gemv_partials(const uint16_t* xh, int rows, int n_sub, const uint16_t
     });
 }
 
+int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, int in_tiles,
+                        int out_tiles, int K, int cb, const uint16_t* suh, int n_sub,
+                        const int32_t* group_sub, const uint16_t* svh, const uint16_t* bias,
+                        uint16_t* y, float* partial, int* counters, GemvPlan plan,
+                        hipStream_t stream) {
+    if (int rc = check_k_cb(K, cb)) return rc;
+    if (!x || !trellis || !y || !partial || !counters) return EXL3_E_NULL_POINTER;
+    if (rows < 1 || rows > kGemvMaxRows || n_sub < 1 || in_tiles < 8 || out_tiles < 8 ||
+        in_tiles % 8 || out_tiles % 8)
+        return EXL3_E_BAD_SHAPE;
+    if (n_sub > 1 && (!group_sub || !suh)) return EXL3_E_BAD_INDEX;
+    if (plan.n_splits < 1 || plan.n_splits > 4 * 65535 || plan.tk_per_split < 1 ||
+        (long long)plan.n_splits * plan.tk_per_split < in_tiles)
+        return EXL3_E_BAD_SHAPE;
+    const int n_groups = out_tiles / 8;
+    const dim3 grid((unsigned)n_groups, (unsigned)((plan.n_splits + 3) / 4));
+    const int mt = rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8;
+    return dispatch_k_cb(K, cb, [&](auto k, auto c) {
+        auto go = [&](auto mtc) {
+            linear_small_kernel<k.value, c.value, mtc.value><<<grid, dim3(256), 0, stream>>>(
+                reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<const half_t*>(x),
+                reinterpret_cast<const half_t*>(suh), reinterpret_cast<const half_t*>(svh),
+                reinterpret_cast<const half_t*>(bias), reinterpret_cast<half_t*>(y), partial,
+                counters, group_sub, in_tiles, out_tiles, rows, n_groups, plan.tk_per_split,
+                plan.n_splits);
+        };
+        switch (mt) {
+            case 1: go(std::integral_constant<int, 1>{}); break;
+            case 2: go(std::integral_constant<int, 2>{}); break;
+            case 4: go(std::integral_constant<int, 4>{}); break;
+            default: go(std::integral_constant<int, 8>{}); break;
+        }
+        return launch_status();
+    });
+}
+
 }  // namespace exl3
 
 EXL3_EXPORT int exl3_gemv_max_rows(void) { return exl3::kGemvMaxRows; }
@@ -197,7 +522,7 @@ EXL3_EXPORT int exl3_gemv_max_rows(void) { return exl3::kGemvMaxRows; }
 EXL3_EXPORT size_t exl3_gemv_workspace_bytes(int rows, int in_tiles, int n_groups) {
     if (rows < 1 || in_tiles < 1 || n_groups < 1) return 0;
     const exl3::GemvPlan plan = exl3::plan_gemv(rows, in_tiles, n_groups);
-    return (size_t)plan.n_splits * rows * n_groups * 128 * sizeof(float);
+    return (size_t)plan.n_partials() * rows * n_groups * 128 * sizeof(float);
 }
 
 EXL3_EXPORT int exl3_gemv_plan(int rows, int in_tiles, int n_groups, int* n_splits,
@@ -205,7 +530,7 @@ EXL3_EXPORT int exl3_gemv_plan(int rows, int in_tiles, int n_groups, int* n_spli
     if (rows < 1 || rows > exl3::kGemvMaxRows || in_tiles < 1 || n_groups < 1)
         return EXL3_E_BAD_SHAPE;
     const exl3::GemvPlan plan = exl3::plan_gemv(rows, in_tiles, n_groups);
-    if (n_splits) *n_splits = plan.n_splits;
+    if (n_splits) *n_splits = plan.n_partials();
     if (tile_rows_per_split) *tile_rows_per_split = plan.tk_per_split;
     return EXL3_OK;
 }
@@ -218,7 +543,7 @@ EXL3_EXPORT int exl3_gemv_partials(const uint16_t* xh, int rows, int n_sub, cons
     using namespace exl3;
     if (rows < 1 || rows > kGemvMaxRows || in_tiles < 1 || n_groups < 1) return EXL3_E_BAD_SHAPE;
     const GemvPlan plan = plan_gemv(rows, in_tiles, n_groups);
-    if (partial_bytes < (size_t)plan.n_splits * rows * n_groups * 128 * sizeof(float))
+    if (partial_bytes < (size_t)plan.n_partials() * rows * n_groups * 128 * sizeof(float))
         return EXL3_E_WORKSPACE;
     return launch_gemv_partials(xh, rows, n_sub, trellis, in_tiles, out_tiles, K, cb, group_sub,
                                 group_tile, n_groups, partial, plan, as_stream(stream));
@@ -233,7 +558,7 @@ EXL3_EXPORT int exl3_gemv(const uint16_t* xh, int rows, int n_sub, const uint16_
     if (rows < 1 || rows > kGemvMaxRows || in_tiles < 1 || n_groups < 1) return EXL3_E_BAD_SHAPE;
     const GemvPlan plan = plan_gemv(rows, in_tiles, n_groups);
     hipStream_t s = as_stream(stream);
-    if (plan.n_splits == 1)
+    if (plan.n_partials() == 1)
         return launch_gemv_partials(xh, rows, n_sub, trellis, in_tiles, out_tiles, K, cb, group_sub,
                                     group_tile, n_groups, y_out, plan, s);
     if (!workspace) return EXL3_E_NULL_POINTER;
@@ -245,6 +570,6 @@ EXL3_EXPORT int exl3_gemv(const uint16_t* xh, int rows, int n_sub, const uint16_
         return rc;
     const size_t n = (size_t)rows * n_groups * 128;
     reduce_partials_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s>>>(partial, y_out, n,
-                                                                                 plan.n_splits);
+                                                                                 plan.n_partials());
     return launch_status();
 }

@@ -78,8 +78,21 @@ __global__ __launch_bounds__(256) void had_post_kernel(const void* __restrict__ 
     float a, b;
     if constexpr (kFp32In) {
         const float* y = reinterpret_cast<const float*>(yv);
-        float2_t acc = *reinterpret_cast<const float2_t*>(y + off);
-        for (int i = 1; i < n_sum; i++) {
+        // slices are loaded eight at a time and added strictly in index order
+        float2_t acc = {0.f, 0.f};
+        int i = 0;
+        for (; i + 8 <= n_sum; i += 8) {
+            float2_t v[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                v[j] = *reinterpret_cast<const float2_t*>(y + (size_t)(i + j) * sum_stride + off);
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                acc.x = acc.x + v[j].x;
+                acc.y = acc.y + v[j].y;
+            }
+        }
+        for (; i < n_sum; i++) {
             const float2_t v = *reinterpret_cast<const float2_t*>(y + (size_t)i * sum_stride + off);
             acc.x = acc.x + v.x;
             acc.y = acc.y + v.y;

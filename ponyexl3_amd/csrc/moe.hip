@@ -178,8 +178,8 @@ static MoeWorkspace moe_workspace(int tokens, int top_k, int D, int H) {
     w.xh_gu = align_up((size_t)slots * 2 * D * 2, 256);
     w.xh_dn = align_up((size_t)slots * H * 2, 256);
     w.tables = align_up((size_t)2 * (w.g_gu + w.g_dn) * sizeof(int), 256);
-    w.part_gu = align_up((size_t)w.plan_gu.n_splits * w.g_gu * 128 * sizeof(float), 256);
-    w.part_dn = align_up((size_t)w.plan_dn.n_splits * w.g_dn * 128 * sizeof(float), 256);
+    w.part_gu = align_up((size_t)w.plan_gu.n_partials() * w.g_gu * 128 * sizeof(float), 256);
+    w.part_dn = align_up((size_t)w.plan_dn.n_partials() * w.g_dn * 128 * sizeof(float), 256);
     w.o_xh_gu = 0;
     w.o_xh_dn = w.o_xh_gu + w.xh_gu;
     w.o_tables = w.o_xh_dn + w.xh_dn;
@@ -242,7 +242,7 @@ EXL3_EXPORT int exl3_moe_forward(const uint16_t* x, int tokens, const int32_t* i
     {
         const int waves = slots * (H / 128);
         moe_glu_kernel<<<dim3((waves + 3) / 4), dim3(256), 0, s>>>(
-            part_gu, w.plan_gu.n_splits, (size_t)w.g_gu * 128, indices,
+            part_gu, w.plan_gu.n_partials(), (size_t)w.g_gu * 128, indices,
             reinterpret_cast<const half_t*>(gu_svh), reinterpret_cast<const half_t*>(dn_suh), xh_dn,
             slots, H, num_experts, activation);
         if (int rc = launch_status()) return rc;
@@ -254,7 +254,7 @@ EXL3_EXPORT int exl3_moe_forward(const uint16_t* x, int tokens, const int32_t* i
     {
         const int waves = slots * (D / 128);
         moe_finish_kernel<<<dim3((waves + 3) / 4), dim3(256), 0, s>>>(
-            part_dn, w.plan_dn.n_splits, (size_t)w.g_dn * 128, indices,
+            part_dn, w.plan_dn.n_partials(), (size_t)w.g_dn * 128, indices,
             reinterpret_cast<const half_t*>(dn_svh), reinterpret_cast<half_t*>(y), slots, D,
             num_experts);
         return launch_status();

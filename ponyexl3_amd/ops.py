@@ -49,6 +49,20 @@ def workspace(device, nbytes: int) -> torch.Tensor:
     return buf
 
 
+_counters: dict = {}
+
+
+def sync_counters(device, n: int) -> torch.Tensor:
+    """Per-device int32 array of group counters for the one-launch layer kernel.
+    Zeroed when created; the kernel leaves it zero, so it is reused as is."""
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    buf = _counters.get(key)
+    if buf is None or buf.numel() < n:
+        buf = torch.zeros(max(int(n), 4096), dtype=torch.int32, device=device)
+        _counters[key] = buf
+    return buf
+
+
 def as_trellis_tensor(trellis, device=None) -> torch.Tensor:
     """numpy/torch uint16|int16 (in_tiles, out_tiles, 16K) -> int16 GPU tensor
     holding the same bits."""
@@ -293,8 +307,10 @@ def inner_gemm(xh, trellis, k: int, cb: int, tn_offset: int = 0, tn_count: int |
     return y
 
 
-def linear_forward(x2d, trellis, k, cb, suh=None, svh=None, bias=None, group_sub=None):
-    """Whole-layer forward on (rows, in) fp16 (``exl3_linear_forward``)."""
+def linear_forward(x2d, trellis, k, cb, suh=None, svh=None, bias=None, group_sub=None,
+                   fused: bool = True):
+    """Whole-layer forward on (rows, in) fp16 (``exl3_linear_forward``).
+    ``fused=False`` selects the three-launch chain for small batches."""
     in_tiles, out_tiles = _trellis_dims(trellis, k)
     _half(x2d, "x")
     if x2d.dim() != 2 or x2d.shape[1] != in_tiles * 16:
@@ -326,9 +342,11 @@ def linear_forward(x2d, trellis, k, cb, suh=None, svh=None, bias=None, group_sub
     lib = _lib.load()
     ws_bytes = int(lib.exl3_linear_workspace_bytes(rows, n_in, n_out, n_sub))
     ws = workspace(x2d.device, ws_bytes)
+    cnt = sync_counters(x2d.device, n_out // 128) if fused else None
     rc = lib.exl3_linear_forward(
         _ptr(x2d), rows, _ptr(trellis), in_tiles, out_tiles, int(k), int(cb), _ptr(suh), n_sub,
-        _ptr(group_sub), _ptr(svh), _ptr(bias), _ptr(y), _ptr(ws), ws.numel(), _stream(),
+        _ptr(group_sub), _ptr(svh), _ptr(bias), _ptr(y), _ptr(ws), ws.numel(), _ptr(cnt),
+        0 if cnt is None else cnt.numel(), _stream(),
     )
     _lib.check(rc, "exl3_linear_forward")
     return y

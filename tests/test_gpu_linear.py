@@ -165,3 +165,25 @@ def test_single_slot_cache_computes_once(cuda):
     s0(torch.zeros((1, 256), dtype=torch.float16, device=cuda))
     assert calls["n"] == 2
     assert s0.out_features == 128 and s0.in_features == 256
+
+
+@pytest.mark.parametrize("rows", [1, 3, 8])
+@pytest.mark.parametrize("k,n_in,n_out", [(4, 512, 384), (3, 1024, 256), (6, 2176, 640), (4, 5120, 1024)])
+def test_one_launch_layer_equals_three_launch_chain(cuda, rows, k, n_in, n_out):
+    """The fused kernel (rotation + GEMV + last-wave reduction + output transform)
+    must reproduce the chained kernels bit for bit, call after call (its group
+    counters have to come back to zero every time)."""
+    from ponyexl3_amd import make_exl3_layer, ops
+
+    layer = make_exl3_layer(k=k, in_features=n_in, out_features=n_out, seed=k + n_in, bias=True)
+    tr = ops.as_trellis_tensor(layer.trellis, cuda)
+    suh = torch.from_numpy(layer.suh).to(cuda)
+    svh = torch.from_numpy(layer.svh).to(cuda)
+    bias = torch.from_numpy(layer.bias).to(cuda)
+    rng = np.random.default_rng(rows)
+    for rep in range(3):
+        x = torch.from_numpy(rng.standard_normal((rows, n_in)).astype(np.float16)).to(cuda)
+        a = ops.linear_forward(x, tr, k, 0, suh, svh, bias, fused=True)
+        b = ops.linear_forward(x, tr, k, 0, suh, svh, bias, fused=False)
+        assert torch.equal(a, b), f"rep {rep}"
+    assert int(ops.sync_counters(cuda, 1).abs().sum()) == 0
