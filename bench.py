@@ -35,6 +35,11 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 K_BITS = 4
 CB = 0
+# HBM bytes moved by the four layer-kernel launches of one step, from two
+# rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE), each scaled
+# by what the same counter reads for a plain copy of known size; see
+# profiles/linear_small_k4_config2_pmc.txt. None until measured.
+TRAFFIC_BYTES_PER_STEP = None
 
 # (name, in, [member out sizes]) of the config-2 layer; several members = sibling-fused
 LAYER_FUSED_QKV = [
@@ -204,7 +209,9 @@ def main():
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
 
-    # ---- roofline of the dominant kernel: the decode GEMV alone, per launch
+    # ---- roofline of the dominant kernel: the one-launch layer kernel (input
+    # Hadamard + decode GEMV + split reduction + output Hadamard), timed per
+    # launch with HIP events on the launch stream
     per_linear = {}
     reps = max(50, min(200, args.steps))
     tot_bytes = tot_ms = 0.0
@@ -213,35 +220,33 @@ def main():
     flush = torch.zeros(1 << 30, dtype=torch.int8, device=dev)
     for j, (name, n_in, outs) in enumerate(LAYER):
         lins = [layers[L][j] for L in range(n_layers)]
-        xh = ops.had128_pre(xs[n_in], lins[0].suh).reshape(1, len(outs), n_in).contiguous()
-        n_splits, _ = ops.gemv_plan(1, n_in // 16, lins[0].n_out // 128)
-        buf = torch.empty((n_splits, 1, lins[0].n_out), dtype=torch.float32, device=dev)
         for r in range(10):
-            ops.inner_gemv_partials(xh, lins[r % n_layers].trellis, K_BITS, CB, lins[0].group_sub, out=buf)
+            lins[r % n_layers].forward(xs[n_in])
         evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
         torch.cuda.synchronize()
         for r in range(reps):
             flush.add_(1)
             evs[r][0].record()
-            ops.inner_gemv_partials(xh, lins[r % n_layers].trellis, K_BITS, CB, lins[0].group_sub, out=buf)
+            lins[r % n_layers].forward(xs[n_in])
             evs[r][1].record()
         torch.cuda.synchronize()
         ms = float(np.mean([a.elapsed_time(b) for a, b in evs]))
         per_linear[name] = {"MB": round(lins[0].bytes / 1e6, 2), "us": round(ms * 1e3, 2),
-                            "GBps": round(lins[0].bytes / ms / 1e6, 1), "n_splits": n_splits}
+                            "GBps": round(lins[0].bytes / ms / 1e6, 1)}
         tot_bytes += lins[0].bytes
         tot_ms += ms
     del flush
     achieved = tot_bytes / tot_ms / 1e6
     roofline = {
         "bound": "hbm",
-        "kernel": "gemv_kernel<K=4, cb=3INST, rows=1>",
+        "kernel": "linear_small_kernel<K=4, cb=3INST, rows=1>",
         "achieved": round(achieved, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
-        "traffic": None,
-        "bytes_per_launch": "in*out*K/8 of the launch's linear(s): sum over the launches of a step / sum of their mean durations",
+        "traffic": TRAFFIC_BYTES_PER_STEP,
+        "bytes_per_launch": "in*out*K/8 of the launch's linear(s); achieved = sum over the launches of a step / "
+                            "sum of their mean durations; traffic = HBM bytes of the same launches (FETCH_SIZE + WRITE_SIZE)",
         "per_linear": per_linear,
     }
 

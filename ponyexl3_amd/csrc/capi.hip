@@ -19,8 +19,10 @@ static LinearWorkspace linear_workspace(int rows, int in_features, int out_featu
     LinearWorkspace w{};
     w.xh_bytes = align_up((size_t)rows * n_sub * in_features * 2, 256);
     if (rows <= kGemvMaxRows) {
-        const GemvPlan plan = plan_gemv(rows, in_features / 16, out_features / 128);
-        w.second_bytes = (size_t)plan.n_partials() * rows * out_features * sizeof(float);
+        const GemvPlan a = plan_gemv(rows, in_features / 16, out_features / 128);
+        const GemvPlan b = plan_linear_small(rows, in_features / 16, out_features / 128);
+        const int n = a.n_partials() > b.n_partials() ? a.n_partials() : b.n_partials();
+        w.second_bytes = (size_t)n * rows * out_features * sizeof(float);
     } else {
         w.second_bytes = (size_t)rows * out_features * 2;
     }
@@ -80,7 +82,8 @@ EXL3_EXPORT int exl3_linear_forward(const uint16_t* x, int rows, const uint16_t*
             // one launch: rotation, GEMV, split reduction and output transform fused
             if (counters_len < (size_t)n_groups) return EXL3_E_WORKSPACE;
             return launch_linear_small(x, rows, trellis, in_tiles, out_tiles, K, cb, suh, n_sub,
-                                       group_sub, svh, bias, y, partial, counters, plan, s);
+                                       group_sub, svh, bias, y, partial, counters,
+                                       plan_linear_small(rows, in_tiles, n_groups), s);
         }
         if (int rc = launch_had_pre(x, rows, in_features, suh, n_sub, xh, s)) return rc;
         if (int rc = launch_gemv_partials(xh, rows, n_sub, trellis, in_tiles, out_tiles, K, cb,

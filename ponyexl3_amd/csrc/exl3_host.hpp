@@ -59,6 +59,7 @@ struct GemvPlan {
     int n_partials() const { return (n_splits + 3) / 4; }
 };
 GemvPlan plan_gemv(int rows, int in_tiles, int n_groups);
+GemvPlan plan_linear_small(int rows, int in_tiles, int n_groups);
 
 // partial: fp32 [plan.n_partials()][rows][128*n_groups]
 int launch_gemv_partials(const uint16_t* xh, int rows, int n_sub, const uint16_t* trellis,

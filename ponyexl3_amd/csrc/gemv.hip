@@ -222,7 +222,7 @@ __global__ __launch_bounds__(256) void linear_small_kernel(
     const bool active = split < n_splits;  // idle waves still take part in the barriers below
     const int sub = group_sub ? group_sub[g] : 0;
     const int in_features = in_tiles * 16;
-    const int tk_begin = active ? split * tk_per_split : 0;
+    const int tk_begin = active ? split * tk_per_split : 0;  // tk_per_split is a multiple of 8
     const int tk_end = active ? min(in_tiles, tk_begin + tk_per_split) : 0;
     const size_t row_words = (size_t)out_tiles * (8 * K);
     const uint32_t* base = trellis + (size_t)g * 8 * (8 * K) + lane * K;
@@ -261,18 +261,29 @@ __global__ __launch_bounds__(256) void linear_small_kernel(
         __builtin_amdgcn_wave_barrier();
     };
 
-    auto consume = [&](const uint32_t (&words)[K], int tk) {
-        if ((tk & 7) == 0 && tk != tk_begin) {  // entering the next Hadamard block
-            rotate_block();
-            if (tk + 8 < tk_end) fetch_block((tk >> 3) + 1);
+    // One pipeline step (see gemv_kernel): neighbour dword of the next slot and
+    // the 16 activations of this tile row (two broadcast LDS reads) are requested
+    // first, then the slot is decoded, multiplied and refilled.
+    struct XTile {
+        uint4_t q[MT][2];
+    };
+    auto load_x = [&](int row_in_block) {
+        XTile t;
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            const uint4_t* xp = reinterpret_cast<const uint4_t*>(&xs[wave][m][row_in_block * 16]);
+            t.q[m][0] = xp[0];
+            t.q[m][1] = xp[1];
         }
-        const LaneWords<K> lw = finish_lane_words<K>(words, lane);
+        return t;
+    };
+    auto consume = [&](const uint32_t (&words)[K], uint32_t prev, const XTile& xt) {
+        const LaneWords<K> lw = make_lane_words<K>(prev, words);
         half2_t wp[16];
         decode_lane<K, CB>(lw, wp);
 #pragma unroll
         for (int m = 0; m < MT; m++) {
-            const uint4_t* xp = reinterpret_cast<const uint4_t*>(&xs[wave][m][(tk & 7) * 16]);
-            const uint4_t x0 = xp[0], x1 = xp[1];
+            const uint4_t x0 = xt.q[m][0], x1 = xt.q[m][1];
             const half2_t xv[8] = {bits_to_half2(x0.x), bits_to_half2(x0.y), bits_to_half2(x0.z),
                                    bits_to_half2(x0.w), bits_to_half2(x1.x), bits_to_half2(x1.y),
                                    bits_to_half2(x1.z), bits_to_half2(x1.w)};
@@ -283,30 +294,35 @@ __global__ __launch_bounds__(256) void linear_small_kernel(
             }
         }
     };
-
+    // Splits are whole Hadamard blocks (8 tile rows), so the block rotation sits
+    // outside the unrolled 8-step pipeline and the LDS offsets of the activations
+    // are compile-time constants.
+    constexpr int kSlots = 4;  // wave-wide loads in flight (divides the 8 steps of a block)
     if (active) {
-        uint32_t buf[kPrefetch][K];
+        uint32_t buf[kSlots][K];
 #pragma unroll
-        for (int s = 0; s < kPrefetch; s++) {
-            const int t = min(tk_begin + s, tk_end - 1);
-            load_lane_words_nt<K>(base + (size_t)t * row_words, buf[s]);
-        }
+        for (int s = 0; s < kSlots; s++)
+            load_lane_words_nt<K>(base + (size_t)min(tk_begin + s, tk_end - 1) * row_words, buf[s]);
         fetch_block(tk_begin >> 3);
-        rotate_block();
-        if (((tk_begin >> 3) + 1) * 8 < tk_end) fetch_block((tk_begin >> 3) + 1);
-
-        int tk0 = tk_begin;
-        for (; tk0 + kPrefetch <= tk_end; tk0 += kPrefetch) {
+        uint32_t prev = neighbour_word(buf[0][K - 1], lane);
+        for (int tkb = tk_begin; tkb < tk_end; tkb += 8) {
+            rotate_block();
+            if (tkb + 8 < tk_end) fetch_block((tkb >> 3) + 1);
 #pragma unroll
-            for (int s = 0; s < kPrefetch; s++) {
-                consume(buf[s], tk0 + s);
-                const int tn = min(tk0 + s + kPrefetch, tk_end - 1);
-                load_lane_words_nt<K>(base + (size_t)tn * row_words, buf[s]);
+            for (int s8 = 0; s8 < 8; s8++) {
+                const int tk = tkb + s8;
+                const int slot = s8 & (kSlots - 1);
+                const uint32_t prev_next =
+                    neighbour_word(buf[(slot + 1) & (kSlots - 1)][K - 1], lane);
+                const XTile xt = load_x(s8);
+                __builtin_amdgcn_sched_barrier(0);
+                consume(buf[slot], prev, xt);
+                const int tn = min(tk + kSlots, tk_end - 1);
+                load_lane_words_nt<K>(base + (size_t)tn * row_words, buf[slot]);
+                __builtin_amdgcn_sched_barrier(0);
+                prev = prev_next;
             }
         }
-#pragma unroll
-        for (int s = 0; s < kPrefetch - 1; s++)
-            if (tk0 + s < tk_end) consume(buf[s], tk0 + s);
     }
 
     // ---- the four waves of the workgroup are summed through LDS in wave order,
@@ -446,6 +462,22 @@ GemvPlan plan_gemv(int rows, int in_tiles, int n_groups) {
     return GemvPlan{n_splits, tk_per_split};
 }
 
+// Plan of the one-launch layer kernel: splits are whole Hadamard blocks (8 tile
+// rows) and every wave gets the same number of blocks where that divides.
+GemvPlan plan_linear_small(int rows, int in_tiles, int n_groups) {
+    (void)rows;
+    static const int kWavesPerSimd = env_int("EXL3_LINEAR_WAVES_PER_SIMD", 12, 1, 16);
+    const int target_waves = 256 * 4 * kWavesPerSimd;
+    const int n_blocks = in_tiles / 8;
+    int max_splits = target_waves / (n_groups > 0 ? n_groups : 1);
+    if (max_splits < 1) max_splits = 1;
+    if (max_splits > n_blocks) max_splits = n_blocks;
+    int blocks_per_split = (n_blocks + max_splits - 1) / max_splits;
+    const int n_splits = (n_blocks + blocks_per_split - 1) / blocks_per_split;
+    blocks_per_split = (n_blocks + n_splits - 1) / n_splits;
+    return GemvPlan{n_splits, blocks_per_split * 8};
+}
+
 int launch_gemv_partials(const uint16_t* xh, int rows, int n_sub, const uint16_t* trellis,
                          int in_tiles, int out_tiles, int K, int cb, const int32_t* group_sub,
                          const int32_t* group_tile, int n_groups, float* partial, GemvPlan plan,
@@ -490,8 +522,8 @@ int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, in
         in_tiles % 8 || out_tiles % 8)
         return EXL3_E_BAD_SHAPE;
     if (n_sub > 1 && (!group_sub || !suh)) return EXL3_E_BAD_INDEX;
-    if (plan.n_splits < 1 || plan.n_splits > 4 * 65535 || plan.tk_per_split < 1 ||
-        (long long)plan.n_splits * plan.tk_per_split < in_tiles)
+    if (plan.n_splits < 1 || plan.n_splits > 4 * 65535 || plan.tk_per_split < 8 ||
+        plan.tk_per_split % 8 || (long long)plan.n_splits * plan.tk_per_split < in_tiles)
         return EXL3_E_BAD_SHAPE;
     const int n_groups = out_tiles / 8;
     const dim3 grid((unsigned)n_groups, (unsigned)((plan.n_splits + 3) / 4));
