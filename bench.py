@@ -38,8 +38,8 @@ CB = 0
 # HBM bytes moved by the four layer-kernel launches of one step, from two
 # rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE), each scaled
 # by what the same counter reads for a plain copy of known size; see
-# profiles/linear_small_k4_config2_pmc.txt. None until measured.
-TRAFFIC_BYTES_PER_STEP = None
+# profiles/linear_small_k4_config2_pmc.txt.
+TRAFFIC_BYTES_PER_STEP = 196_178_842
 
 # (name, in, [member out sizes]) of the config-2 layer; several members = sibling-fused
 LAYER_FUSED_QKV = [
