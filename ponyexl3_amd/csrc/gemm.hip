@@ -107,21 +107,40 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const uint32_t* __restrict
     const int fr = lane & 15, fk = (lane >> 4) * 8;
     for (int ks = 0; ks < ksteps; ks++) {
         if (ks + 1 < ksteps) load_global(ks + 1);
+        // MFMA phase. Fragment reads are software-pipelined by hand: the A
+        // fragments of the next pair of 16-row tiles are requested before the
+        // eight MFMAs of the current pair are issued, so LDS latency hides
+        // behind 128 cycles of matrix work instead of stalling every 4 MFMAs.
 #pragma unroll
         for (int kk = 0; kk < 2; kk++) {
             half8_t bf[4];
+            half8_t af[2][2];
+            auto load_a = [&](int i) {
+                return *reinterpret_cast<const half8_t*>(
+                    &a_s[(wm * 128 + i * 16 + fr) * LDS_LD + kk * 32 + fk]);
+            };
 #pragma unroll
             for (int j = 0; j < 4; j++)
                 bf[j] = *reinterpret_cast<const half8_t*>(
                     &b_s[(wn * 64 + j * 16 + fr) * LDS_LD + kk * 32 + fk]);
+            af[0][0] = load_a(0);
+            af[0][1] = load_a(1);
+            __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);  // 4 B + 2 A fragment reads
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const half8_t af = *reinterpret_cast<const half8_t*>(
-                    &a_s[(wm * 128 + i * 16 + fr) * LDS_LD + kk * 32 + fk]);
+            for (int ip = 0; ip < 4; ip++) {
+                if (ip < 3) {
+                    af[(ip + 1) & 1][0] = load_a(2 * ip + 2);
+                    af[(ip + 1) & 1][1] = load_a(2 * ip + 3);
+                }
 #pragma unroll
-                for (int j = 0; j < 4; j++)
-                    acc[i][j] =
-                        __builtin_amdgcn_mfma_f32_16x16x32_f16(bf[j], af, acc[i][j], 0, 0, 0);
+                for (int h = 0; h < 2; h++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        acc[2 * ip + h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                            bf[j], af[ip & 1][h], acc[2 * ip + h][j], 0, 0, 0);
+                // pin the order: next pair's two reads first, then this pair's eight MFMAs
+                if (ip < 3) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
             }
         }
         __syncthreads();
