@@ -140,10 +140,20 @@ int exl3_gemv_partials(const uint16_t *xh, int rows, int n_sub, const uint16_t *
  *   xh      fp16 [rows][ldx] (ldx >= in, elements)
  *   y_out   fp16 [rows][ldy] written at column offset 0 (ldy >= out); the fp32
  *           accumulator is rounded once (the cast at ponyexl3/ref/forward.py:41)
+ *   workspace  device scratch of exl3_gemm_workspace_bytes(rows, in_tiles, tn_count)
+ *           bytes, 16-byte aligned, for the fp32 partial tiles of block tiles that
+ *           are split along the reduction dimension to fill the last round of
+ *           CUs (the reference's small-batch kernels split K for the same reason,
+ *           ponyexl3/mlx/gemv_metal.py:1405-1414).
+ *           NULL or too small: no tile is split (slower on some shapes, same result
+ *           up to the order of fp32 additions).
  */
 int exl3_gemm(const uint16_t *xh, int rows, size_t ldx, const uint16_t *trellis, int in_tiles,
               int out_tiles, int K, int cb, int tn_offset, int tn_count, uint16_t *y_out,
-              size_t ldy, void *stream);
+              size_t ldy, void *workspace, size_t workspace_bytes, void *stream);
+
+/* Scratch bytes exl3_gemm can use for this shape (0 when no tile would be split). */
+size_t exl3_gemm_workspace_bytes(int rows, int in_tiles, int tn_count);
 
 /*
  * Whole layer forward (ponyexl3/ref/forward.py:14-49, EXL3Linear.__call__ at

@@ -9,10 +9,12 @@ namespace exl3 {
 //   [0, xh_bytes)            xh  fp16 [rows][n_sub][in]
 //   [xh_bytes, ...)          rows <= kGemvMaxRows: fp32 split-K partials
 //                            otherwise:            fp16 y [rows][out]
+//   then (rows > kGemvMaxRows) the fp32 partial tiles of the prefill GEMM
 struct LinearWorkspace {
     size_t xh_bytes;
     size_t second_bytes;
-    size_t total() const { return xh_bytes + second_bytes; }
+    size_t gemm_bytes;
+    size_t total() const { return xh_bytes + second_bytes + gemm_bytes; }
 };
 
 static LinearWorkspace linear_workspace(int rows, int in_features, int out_features, int n_sub) {
@@ -25,6 +27,7 @@ static LinearWorkspace linear_workspace(int rows, int in_features, int out_featu
         w.second_bytes = (size_t)n * rows * out_features * sizeof(float);
     } else {
         w.second_bytes = (size_t)rows * out_features * 2;
+        w.gemm_bytes = align_up(gemm_workspace_bytes(rows, in_features / 16, out_features / 16), 256);
     }
     w.second_bytes = align_up(w.second_bytes, 256);
     return w;
@@ -98,7 +101,8 @@ EXL3_EXPORT int exl3_linear_forward(const uint16_t* x, int rows, const uint16_t*
     uint16_t* ytmp = reinterpret_cast<uint16_t*>(second);
     if (n_sub == 1) {
         if (int rc = launch_gemm(xh, rows, (size_t)in_features, trellis, in_tiles, out_tiles, K, cb,
-                                 0, out_tiles, ytmp, (size_t)out_features, s))
+                                 0, out_tiles, ytmp, (size_t)out_features,
+                                 second + ws.second_bytes, ws.gemm_bytes, s))
             return rc;
     } else {
         return EXL3_E_UNSUPPORTED;  // fused groups run their members one by one on the host side

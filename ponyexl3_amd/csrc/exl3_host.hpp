@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "../../include/exl3_hip.h"
 
@@ -81,10 +82,32 @@ int launch_had_pre(const uint16_t* x, int rows, int n, const uint16_t* suh, int 
 int launch_had_post(const void* y, int y_is_fp32, int n_sum, size_t sum_stride, int rows, int n,
                     const uint16_t* svh, const uint16_t* bias, uint16_t* out, hipStream_t stream);
 
+// Tile schedule of the prefill GEMM: block tiles of (32*mi) rows x 256 columns are
+// dealt to the CUs in rounds; the `split_tiles` tiles of a partly filled last
+// round are cut into `split` reduction ranges of `ksteps_per_split` 64-deep steps
+// whose fp32 partial tiles a second kernel adds up.
+struct GemmPlan {
+    int mi;  // 16-row accumulator tiles per wave: 8 (256-row blocks) or 2 (64-row blocks)
+    int n_row_blocks, n_col_blocks;
+    int full_tiles, split_tiles;
+    int split, ksteps_per_split;
+};
+GemmPlan plan_gemm(int rows, int in_tiles, int tn_count, bool allow_split);
+size_t gemm_workspace_bytes(int rows, int in_tiles, int tn_count);
+
+// workspace may be NULL (or too small): then no tile is split.
 int launch_gemm(const uint16_t* xh, int rows, size_t ldx, const uint16_t* trellis, int in_tiles,
                 int out_tiles, int K, int cb, int tn_offset, int tn_count, uint16_t* y_out,
-                size_t ldy, hipStream_t stream);
+                size_t ldy, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Integer tuning knob from the environment, clamped to [lo, hi].
+inline int env_int(const char* name, int dflt, int lo, int hi) {
+    const char* v = getenv(name);
+    if (!v || !*v) return dflt;
+    const int x = atoi(v);
+    return x < lo ? lo : (x > hi ? hi : x);
+}
 
 }  // namespace exl3

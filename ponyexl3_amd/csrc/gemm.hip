@@ -1,19 +1,35 @@
 // Prefill GEMM: y = xh @ W_inner with the trellis decoded into LDS and
 // contracted on fp16 MFMA (v_mfma_f32_16x16x32_f16), fp32 accumulation.
 //
-// Tiling (one workgroup = 4 wavefronts, two workgroups fit a CU so the decode
-// phase of one overlaps the MFMA phase of the other):
-//   block tile   BM x BN = 256 rows x 128 columns, BK = 64 (four tile rows)
-//   wave tile    128 x 64 -> 8 x 4 accumulator tiles of 16x16 (128 VGPRs)
-//   per BK step  wave w decodes tile row k0/16 + w of the block's 8 tile columns
-//                (one 256*K-byte wave-wide load, 32 codewords per lane) and
-//                writes fp16 columns into the B tile; all threads copy the
-//                256 x 64 activation tile into the A tile.
-// LDS rows (64 halfs) are padded to 72 halfs so that 16-byte fragment reads of
-// 8 consecutive rows touch all 32 banks once.
+// One workgroup = 8 wavefronts (2 per SIMD), one workgroup per CU.
+//   block tile   BM x 256 columns, BK = 64 (four tile rows); BM = 256 (MI = 8) or
+//                64 (MI = 2, small batches: less padding work per decoded tile)
+//   wave tile    (BM/2) x 64 -> MI x 4 accumulator tiles of 16x16
+//   LDS          two stages of A [BM][64] and B [256][64] fp16 (128 KiB at MI = 8):
+//                stage s^1 is filled while stage s is contracted, one barrier per
+//                64-deep step
+//   B fill       wave w decodes tile row (w & 3) of the 8 tile columns of half
+//                (w >> 2): one 256*K-byte wave-wide load, 32 codewords per lane
+//   A fill       global -> LDS direct loads (global_load_lds_dwordx4): lane l of a
+//                wave-wide load lands at byte 16*l of a 1 KiB block = 8 rows of 64
+//                halfs, so no VGPRs and no ds_write are spent on activations
+// LDS rows are 64 halfs (128 B) unpadded; the 16-byte chunk c of row r is stored
+// at chunk c ^ (((r >> 1) & 3) << 1). Measured on gfx950 this makes the b128
+// fragment reads (16 rows x 4 chunks per wave) run at the same ~190 B/clk/CU as a
+// padded layout while keeping each 8-row block contiguous for the direct loads.
+//
+// Decode work is spread over the MFMA stream: after each group of 8 MFMAs a wave
+// decodes 32/MI codewords, which the hardware issues in the shadow of the matrix
+// pipe (about two VALU instructions per MFMA are free).
 //
 // The MFMA is issued as D^T = B^T A^T (weights as the first operand), so a lane
-// ends up with 4 consecutive output columns of one row and stores 8 bytes.
+// ends up with 4 consecutive output columns of one row.
+//
+// Tail handling: tiles are dealt to CUs in rounds. The tiles of a last, partly
+// filled round are split along the reduction dimension into `split` ranges so
+// that the round costs 1/split of a tile time; those workgroups write fp32
+// partial tiles to a workspace and a small second kernel adds them in a fixed
+// order and rounds once to fp16.
 //
 // Replaces the rows > 16 ladder of EXL3Linear.__call__
 // (ponyexl3/mlx/exl3_linear.py:137-161) and the decode-into-threadgroup-memory
@@ -23,155 +39,364 @@
 
 namespace exl3 {
 
-constexpr int BM = 256, BN = 128, BK = 64;
-constexpr int LDS_LD = BK + 8;  // halfs per padded LDS row
+constexpr int kGemmBN = 256;       // columns per block tile
+constexpr int kGemmThreads = 512;  // 8 waves
+constexpr int kGemmStageB = kGemmBN * 64;
 
-template <int K, int CB>
-__global__ __launch_bounds__(256, 2) void gemm_kernel(const uint32_t* __restrict__ trellis,
-                                                      const half_t* __restrict__ xh,
-                                                      half_t* __restrict__ y, int rows,
-                                                      size_t ldx, size_t ldy, int in_tiles,
-                                                      int out_tiles, int tn_offset) {
-    __shared__ __attribute__((aligned(16))) half_t a_s[BM * LDS_LD];
-    __shared__ __attribute__((aligned(16))) half_t b_s[BN * LDS_LD];
+__device__ __forceinline__ int lds_chunk_swizzle(int row) { return ((row >> 1) & 3) << 1; }
 
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;  // wave tile origin: rows wm*128, cols wn*64
-    const int m0 = blockIdx.y * BM;
-    const int g = blockIdx.x;  // 128-column group inside the slice
-    const int tn0 = tn_offset + g * 8;
+// Work unit `unit` of the launch -> tile and reduction range.
+struct GemmWork {
+    int tile, k_begin, k_end, partial_unit;  // partial_unit < 0: direct fp16 output
+};
 
-    float4_t acc[8][4];
-#pragma unroll
-    for (int i = 0; i < 8; i++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+__device__ __forceinline__ GemmWork gemm_work(int unit, int full_tiles, int split,
+                                              int ksteps_per_split, int ksteps) {
+    GemmWork w;
+    if (unit < full_tiles) {
+        w.tile = unit;
+        w.k_begin = 0;
+        w.k_end = ksteps;
+        w.partial_unit = -1;
+    } else {
+        const int r = unit - full_tiles;
+        w.tile = full_tiles + r / split;
+        const int sp = r % split;
+        w.k_begin = sp * ksteps_per_split;
+        w.k_end = min(ksteps, w.k_begin + ksteps_per_split);
+        w.partial_unit = split > 1 ? r : -1;
+    }
+    return w;
+}
 
+template <int K, int CB, int MI>
+__global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
+    const uint32_t* __restrict__ trellis, const half_t* __restrict__ xh, half_t* __restrict__ y,
+    float* __restrict__ partial, int rows, size_t ldx, size_t ldy, int in_tiles, int out_tiles,
+    int tn_offset, int tn_count, int n_row_blocks, int full_tiles, int split,
+    int ksteps_per_split) {
+    extern __shared__ __attribute__((aligned(16))) half_t smem[];
+    constexpr int BM = 32 * MI;
+    constexpr int STAGE_A = BM * 64, STAGE_B = kGemmStageB;
+    half_t* a_s = smem;
+    half_t* b_s = smem + 2 * STAGE_A;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 2, wn = wave & 3;  // wave tile origin: rows wm*16*MI, columns wn*64
+    const GemmWork work = gemm_work(blockIdx.x, full_tiles, split, ksteps_per_split, in_tiles / 4);
+    const int g = work.tile / n_row_blocks;  // 256-column block inside the slice
+    const int m0 = (work.tile % n_row_blocks) * BM;
+    const int k_begin = work.k_begin, k_last = work.k_end - 1;
+    const int nsteps = work.k_end - work.k_begin;
+
+    // ---- fill side: what this wave brings into LDS every step ----
+    const int tr = wave & 3;
+    // the last column block of a slice may hold only 8 tile columns: its upper half
+    // re-decodes the lower half's tiles (results never stored)
+    const int ch = (g * 16 + 8 < tn_count) ? (wave >> 2) : 0;
     const size_t row_words = (size_t)out_tiles * (8 * K);
-    const uint32_t* tbase = trellis + (size_t)tn0 * (8 * K) + lane * K;
-
-    // A-tile copy assignment: chunk c = tid + 256*i covers row c/8, halfs (c%8)*8..+7
-    uint4_t a_reg[8];
-    uint32_t w_reg[K];
-
-    auto load_global = [&](int kstep) {
-        const uint32_t* p = tbase + (size_t)(kstep * 4 + wave) * row_words;
+    const uint32_t* tbase = trellis + (size_t)(tn_offset + g * 16 + ch * 8) * (8 * K) +
+                            (size_t)tr * row_words + lane * K;
+    const size_t t_step = 4 * row_words;
+    int b_w[2];  // half offsets of the lane's two columns inside a B stage (chunk 2*tr)
 #pragma unroll
-        for (int i = 0; i < K; i++) w_reg[i] = p[i];
+    for (int cs = 0; cs < 2; cs++) {
+        const int n = (wave >> 2) * 128 + (lane >> 3) * 16 + (lane & 7) + 8 * cs;
+        b_w[cs] = n * 64 + ((2 * tr) ^ lds_chunk_swizzle(n)) * 8;
+    }
+    // A tile: wave w copies rows w*4*MI .. +4*MI-1 with MI/2 direct loads of 8 rows each
+    const char* abase = reinterpret_cast<const char*>(xh + (size_t)m0 * ldx);
+    uint32_t a_off[MI / 2];
+    {
+        const int rl = lane >> 3;
+        const int c = (lane & 7) ^ lds_chunk_swizzle(rl);
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int c = tid + 256 * i;
-            const int r = m0 + (c >> 3);
-            if (r < rows)
-                a_reg[i] = *reinterpret_cast<const uint4_t*>(xh + (size_t)r * ldx +
-                                                             (size_t)kstep * BK + (c & 7) * 8);
-            else
-                a_reg[i] = uint4_t{0u, 0u, 0u, 0u};
-        }
-    };
-
-    auto store_lds = [&]() {
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int c = tid + 256 * i;
-            *reinterpret_cast<uint4_t*>(&a_s[(c >> 3) * LDS_LD + (c & 7) * 8]) = a_reg[i];
-        }
-        const LaneWords<K> lw = finish_lane_words<K>(w_reg, lane);
-        half2_t wp[16];
-        decode_lane<K, CB>(lw, wp);
-        const int col = (lane >> 3) * 16 + (lane & 7);
-#pragma unroll
-        for (int cs = 0; cs < 2; cs++) {
-            half_t* dst = &b_s[(col + 8 * cs) * LDS_LD + wave * 16];
-            uint4_t v0, v1;
-            v0.x = half2_to_bits(wp[8 * cs + 0]);
-            v0.y = half2_to_bits(wp[8 * cs + 1]);
-            v0.z = half2_to_bits(wp[8 * cs + 2]);
-            v0.w = half2_to_bits(wp[8 * cs + 3]);
-            v1.x = half2_to_bits(wp[8 * cs + 4]);
-            v1.y = half2_to_bits(wp[8 * cs + 5]);
-            v1.z = half2_to_bits(wp[8 * cs + 6]);
-            v1.w = half2_to_bits(wp[8 * cs + 7]);
-            *reinterpret_cast<uint4_t*>(dst) = v0;
-            *reinterpret_cast<uint4_t*>(dst + 8) = v1;
-        }
-    };
-
-    const int ksteps = in_tiles / 4;
-    load_global(0);
-    store_lds();
-    __syncthreads();
-
-    const int fr = lane & 15, fk = (lane >> 4) * 8;
-    for (int ks = 0; ks < ksteps; ks++) {
-        if (ks + 1 < ksteps) load_global(ks + 1);
-        // MFMA phase. Fragment reads are software-pipelined by hand: the A
-        // fragments of the next pair of 16-row tiles are requested before the
-        // eight MFMAs of the current pair are issued, so LDS latency hides
-        // behind 128 cycles of matrix work instead of stalling every 4 MFMAs.
-#pragma unroll
-        for (int kk = 0; kk < 2; kk++) {
-            half8_t bf[4];
-            half8_t af[2][2];
-            auto load_a = [&](int i) {
-                return *reinterpret_cast<const half8_t*>(
-                    &a_s[(wm * 128 + i * 16 + fr) * LDS_LD + kk * 32 + fk]);
-            };
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-                bf[j] = *reinterpret_cast<const half8_t*>(
-                    &b_s[(wn * 64 + j * 16 + fr) * LDS_LD + kk * 32 + fk]);
-            af[0][0] = load_a(0);
-            af[0][1] = load_a(1);
-            __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);  // 4 B + 2 A fragment reads
-#pragma unroll
-            for (int ip = 0; ip < 4; ip++) {
-                if (ip < 3) {
-                    af[(ip + 1) & 1][0] = load_a(2 * ip + 2);
-                    af[(ip + 1) & 1][1] = load_a(2 * ip + 3);
-                }
-#pragma unroll
-                for (int h = 0; h < 2; h++)
-#pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        acc[2 * ip + h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                            bf[j], af[ip & 1][h], acc[2 * ip + h][j], 0, 0, 0);
-                // pin the order: next pair's two reads first, then this pair's eight MFMAs
-                if (ip < 3) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
-            }
-        }
-        __syncthreads();
-        if (ks + 1 < ksteps) {
-            store_lds();
-            __syncthreads();
+        for (int i = 0; i < MI / 2; i++) {
+            int r = wave * (4 * MI) + i * 8 + rl;
+            if (m0 + r >= rows) r = rows - 1 - m0;  // rows past the end are never stored
+            a_off[i] = (uint32_t)((size_t)r * ldx * 2 + c * 16);
         }
     }
+    uint32_t w_reg[2][K];
 
-    // acc[i][j] is D^T: lane holds columns n = 4*(lane/16)+0..3 of row m = lane%16
+    auto load_w = [&](int kstep, auto slot) {
+        constexpr int s = decltype(slot)::value;
+        const uint32_t* p = tbase + (size_t)kstep * t_step;
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int r = m0 + wm * 128 + i * 16 + fr;
-        if (r < rows) {
+        for (int i = 0; i < K; i++) w_reg[s][i] = __builtin_nontemporal_load(p + i);
+    };
+    auto load_a = [&](int kstep, int stage) {
+        const char* ab = abase + (size_t)kstep * 128;
+        half_t* as = a_s + stage * STAGE_A + wave * (4 * MI) * 64;
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int c = g * 128 + wn * 64 + j * 16 + (lane >> 4) * 4;
-                half4_t o;
-                o.x = (half_t)acc[i][j].x;
-                o.y = (half_t)acc[i][j].y;
-                o.z = (half_t)acc[i][j].z;
-                o.w = (half_t)acc[i][j].w;
-                *reinterpret_cast<half4_t*>(y + (size_t)r * ldy + c) = o;
+        for (int i = 0; i < MI / 2; i++)
+            __builtin_amdgcn_global_load_lds(
+                (const void __attribute__((address_space(1)))*)(ab + a_off[i]),
+                (void __attribute__((address_space(3)))*)(as + i * 8 * 64), 16, 0, 0);
+    };
+    // Pair pi (0..15) of a lane = codewords 2pi, 2pi+1 = input rows (2j, 2j+1) of
+    // column u + 8*cs with cs = (pi>>1)&1, j = (pi>>2) + 4*(pi&1). The four pairs
+    // {2cs + hh + 4t, t = 0..3} are the 8 consecutive rows 8hh..8hh+7 of column cs:
+    // one 16-byte store. Element e = 4*quad + t of the decode order.
+    auto decode_element = [&](const LaneWords<K>& lw, auto e_c, uint4_t& quad, half_t* bdst) {
+        constexpr int e = decltype(e_c)::value;
+        constexpr int q = e >> 2, t = e & 3;
+        constexpr int cs = q >> 1, hh = q & 1;
+        constexpr int pi = 2 * cs + hh + 4 * t;
+        const uint32_t d = half2_to_bits(
+            decode_pair<CB>(lane_codeword<K, 2 * pi>(lw), lane_codeword<K, 2 * pi + 1>(lw)));
+        if constexpr (t == 0) quad.x = d;
+        if constexpr (t == 1) quad.y = d;
+        if constexpr (t == 2) quad.z = d;
+        if constexpr (t == 3) {
+            quad.w = d;
+            *reinterpret_cast<uint4_t*>(bdst + b_w[cs] + 8 * hh) = quad;
+        }
+    };
+
+    // ---- MFMA side ----
+    float4_t acc[MI][4];
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+    const int fr = lane & 15;
+    // half offset of the lane's 16-byte chunk for the first 32 k; the second 32 k flip chunk bit 2
+    const int pk0 = ((lane >> 4) ^ lds_chunk_swizzle(fr)) * 8;
+    const half_t* a_frag = a_s + (wm * (16 * MI) + fr) * 64;
+    const half_t* b_frag = b_s + (wn * 64 + fr) * 64;
+
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    auto clamp_k = [&](int k) { return k < k_last ? k : k_last; };
+
+    // prologue: stage 0 <- step 0; slot 1 <- step 1, slot 0 <- step 2
+    {
+        load_w(k_begin, S0{});
+        load_a(k_begin, 0);
+        load_w(clamp_k(k_begin + 1), S1{});
+        const LaneWords<K> lw = finish_lane_words<K>(w_reg[0], lane);
+        uint4_t quad;
+        static_for<0, 16>([&](auto e) { decode_element(lw, e, quad, b_s); });
+        load_w(clamp_k(k_begin + 2), S0{});
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    // Step i contracts stage i&1 and fills stage (i+1)&1 with step i+1, whose
+    // trellis words sit in slot (i+1)&1; that slot is then refilled with step i+3.
+    auto step = [&](int i, auto slot) {
+        constexpr int s = decltype(slot)::value;
+        const int stage = i & 1;
+        const int k = k_begin + i;
+        load_a(clamp_k(k + 1), stage ^ 1);
+        const LaneWords<K> lw = finish_lane_words<K>(w_reg[s], lane);
+        load_w(clamp_k(k + 3), slot);
+        const half_t* as = a_frag + stage * STAGE_A;
+        const half_t* bs = b_frag + stage * STAGE_B;
+        half_t* bdst = b_s + (stage ^ 1) * STAGE_B;
+        uint4_t quad;
+        half8_t bf[4];
+        half8_t af[3][2];
+        auto lda = [&](int kk, int ii) {
+            return *reinterpret_cast<const half8_t*>(as + ii * 16 * 64 + (pk0 ^ (kk * 32)));
+        };
+        auto ldb = [&](int kk, int j) {
+            return *reinterpret_cast<const half8_t*>(bs + j * 16 * 64 + (pk0 ^ (kk * 32)));
+        };
+        // MFMA group gi = 8 MFMAs = two 16-row tiles x four 16-column tiles x 32 k;
+        // MI groups per step, A fragments are requested two groups ahead.
+        constexpr int G = MI;
+        constexpr int GH = MI / 2;  // groups per 32-deep half
+        auto lda_group = [&](auto gi_c) {
+            constexpr int gi = decltype(gi_c)::value;
+            af[gi % 3][0] = lda(gi / GH, 2 * (gi % GH));
+            af[gi % 3][1] = lda(gi / GH, 2 * (gi % GH) + 1);
+        };
+#pragma unroll
+        for (int j = 0; j < 4; j++) bf[j] = ldb(0, j);
+        lda_group(std::integral_constant<int, 0>{});
+        lda_group(std::integral_constant<int, 1>{});
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<0, G>([&](auto gi_c) {
+            constexpr int gi = decltype(gi_c)::value;
+            constexpr int ip = gi % GH;
+            if constexpr (gi + 2 < G) lda_group(std::integral_constant<int, gi + 2>{});
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    acc[2 * ip + h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                        bf[j], af[gi % 3][h], acc[2 * ip + h][j], 0, 0, 0);
+            if constexpr (gi == GH - 1) {  // weights of the second half, once the first half is issued
+#pragma unroll
+                for (int j = 0; j < 4; j++) bf[j] = ldb(1, j);
+            }
+            static_for<gi * (16 / G), (gi + 1) * (16 / G)>(
+                [&](auto e) { decode_element(lw, e, quad, bdst); });
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the direct loads of stage^1 have landed
+        __syncthreads();
+    };
+
+    int i = 0;
+    for (; i + 1 < nsteps; i += 2) {
+        step(i, S1{});
+        step(i + 1, S0{});
+    }
+    if (i < nsteps) step(i, S1{});
+
+    // acc[i][j] is D^T: lane holds columns 4*(lane/16)+0..3 of row lane%16
+    const int col0 = g * kGemmBN + wn * 64 + (lane >> 4) * 4;
+    if (g * kGemmBN + wn * 64 >= tn_count * 16) return;  // upper half of a half-width last block
+    if (work.partial_unit < 0) {
+#pragma unroll
+        for (int ii = 0; ii < MI; ii++) {
+            const int r = m0 + wm * (16 * MI) + ii * 16 + fr;
+            if (r < rows) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    half4_t o;
+                    o.x = (half_t)acc[ii][j].x;
+                    o.y = (half_t)acc[ii][j].y;
+                    o.z = (half_t)acc[ii][j].z;
+                    o.w = (half_t)acc[ii][j].w;
+                    *reinterpret_cast<half4_t*>(y + (size_t)r * ldy + col0 + j * 16) = o;
+                }
+            }
+        }
+    } else {
+        float* pt = partial + (size_t)work.partial_unit * (BM * kGemmBN);
+#pragma unroll
+        for (int ii = 0; ii < MI; ii++) {
+            const int rl = wm * (16 * MI) + ii * 16 + fr;
+            if (m0 + rl < rows) {
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    *reinterpret_cast<float4_t*>(pt + rl * kGemmBN + wn * 64 + (lane >> 4) * 4 +
+                                                 j * 16) = acc[ii][j];
             }
         }
     }
 }
 
+// Sums the `split` fp32 partial tiles of every split tile in index order and
+// rounds once to fp16. grid = (split tiles, BM/8): a workgroup of 256 threads
+// finishes 8 rows x 256 columns, one float4 per thread and range.
+template <int MI>
+__global__ __launch_bounds__(256) void gemm_fixup_kernel(const float* __restrict__ partial,
+                                                         half_t* __restrict__ y, int rows,
+                                                         size_t ldy, int tn_count,
+                                                         int n_row_blocks, int full_tiles,
+                                                         int split) {
+    constexpr int BM = 32 * MI;
+    const int tile = full_tiles + blockIdx.x;
+    const int g = tile / n_row_blocks;
+    const int m0 = (tile % n_row_blocks) * BM;
+    const int c4 = (threadIdx.x & 63) * 4;
+    if (g * kGemmBN + c4 >= tn_count * 16) return;
+    const float* p0 = partial + (size_t)blockIdx.x * split * (BM * kGemmBN);
+#pragma unroll
+    for (int it = 0; it < 2; it++) {
+        const int rl = blockIdx.y * 8 + it * 4 + (threadIdx.x >> 6);
+        if (m0 + rl >= rows) return;
+        const float* p = p0 + rl * kGemmBN + c4;
+        float4_t s = *reinterpret_cast<const float4_t*>(p);
+#pragma unroll 4
+        for (int sp = 1; sp < split; sp++)
+            s = s + *reinterpret_cast<const float4_t*>(p + (size_t)sp * (BM * kGemmBN));
+        half4_t o;
+        o.x = (half_t)s.x;
+        o.y = (half_t)s.y;
+        o.z = (half_t)s.z;
+        o.w = (half_t)s.w;
+        *reinterpret_cast<half4_t*>(y + (size_t)(m0 + rl) * ldy + g * kGemmBN + c4) = o;
+    }
+}
+
+static int gemm_slots() {
+    // one workgroup per CU; the count only shapes the schedule, never the result of a tile
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+            n < 1)
+            n = 256;
+        return n;
+    }();
+    return env_int("EXL3_GEMM_SLOTS", cus, 1, 4096);
+}
+
+GemmPlan plan_gemm(int rows, int in_tiles, int tn_count, bool allow_split) {
+    GemmPlan p{};
+    p.mi = rows <= 64 ? 2 : 8;
+    const int bm = 32 * p.mi;
+    p.n_row_blocks = (rows + bm - 1) / bm;
+    p.n_col_blocks = (tn_count + 15) / 16;
+    const long long tiles = (long long)p.n_row_blocks * p.n_col_blocks;
+    const int ksteps = in_tiles / 4;
+    const int slots = gemm_slots();
+    p.full_tiles = (int)(tiles / slots * slots);
+    p.split = 1;
+    p.ksteps_per_split = ksteps;
+    const int rem = (int)(tiles - p.full_tiles);
+    if (allow_split && rem > 0) {
+        // Cost of the last round in tile times: its workgroups run in
+        // ceil(rem*s/slots) waves of 1/s tile each, and every range also writes (and
+        // the fix-up reads) one fp32 tile, about the time of 8 steps.
+        const int max_split = env_int("EXL3_GEMM_MAX_SPLIT", 8, 1, 64);
+        const double partial_cost = 8.0 / ksteps;
+        double best = 1.0;
+        for (int s = 2; s <= max_split && ksteps / s >= 4; s++) {
+            const int kps = (ksteps + s - 1) / s;
+            if ((ksteps + kps - 1) / kps != s) continue;  // some range would be empty
+            const double cost =
+                (double)(((long long)rem * s + slots - 1) / slots) * (1.0 / s + partial_cost);
+            if (cost < best - 1e-9) {
+                best = cost;
+                p.split = s;
+                p.ksteps_per_split = kps;
+            }
+        }
+    }
+    if (p.split == 1) p.full_tiles = (int)tiles;  // nothing to fix up
+    p.split_tiles = (int)(tiles - p.full_tiles);
+    return p;
+}
+
+size_t gemm_workspace_bytes(int rows, int in_tiles, int tn_count) {
+    const GemmPlan p = plan_gemm(rows, in_tiles, tn_count, true);
+    return (size_t)p.split_tiles * p.split * (32 * p.mi) * kGemmBN * sizeof(float);
+}
+
+template <int K, int CB, int MI>
+static int launch_gemm_mi(const GemmPlan& p, const uint16_t* xh, int rows, size_t ldx,
+                          const uint16_t* trellis, int in_tiles, int out_tiles, int tn_offset,
+                          int tn_count, uint16_t* y_out, size_t ldy, float* partial,
+                          hipStream_t stream) {
+    constexpr size_t lds = (2 * (size_t)(32 * MI) * 64 + 2 * (size_t)kGemmStageB) * sizeof(half_t);
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_kernel<K, CB, MI>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return EXL3_E_LAUNCH;
+    const unsigned units = (unsigned)(p.full_tiles + p.split_tiles * p.split);
+    gemm_kernel<K, CB, MI><<<dim3(units), dim3(kGemmThreads), lds, stream>>>(
+        reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<const half_t*>(xh),
+        reinterpret_cast<half_t*>(y_out), partial, rows, ldx, ldy, in_tiles, out_tiles, tn_offset,
+        tn_count, p.n_row_blocks, p.full_tiles, p.split, p.ksteps_per_split);
+    if (int rc = launch_status()) return rc;
+    if (p.split_tiles > 0) {
+        gemm_fixup_kernel<MI><<<dim3((unsigned)p.split_tiles, 4 * MI), dim3(256), 0, stream>>>(
+            partial, reinterpret_cast<half_t*>(y_out), rows, ldy, tn_count, p.n_row_blocks,
+            p.full_tiles, p.split);
+        return launch_status();
+    }
+    return EXL3_OK;
+}
+
 int launch_gemm(const uint16_t* xh, int rows, size_t ldx, const uint16_t* trellis, int in_tiles,
                 int out_tiles, int K, int cb, int tn_offset, int tn_count, uint16_t* y_out,
-                size_t ldy, hipStream_t stream) {
+                size_t ldy, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     if (int rc = check_k_cb(K, cb)) return rc;
     if (!xh || !trellis || !y_out) return EXL3_E_NULL_POINTER;
     if (rows < 1 || in_tiles < 4 || in_tiles % 4 || tn_offset < 0 || tn_count < 8 ||
@@ -180,22 +405,37 @@ int launch_gemm(const uint16_t* xh, int rows, size_t ldx, const uint16_t* trelli
         return EXL3_E_BAD_SHAPE;
     if ((reinterpret_cast<uintptr_t>(xh) & 15) || (reinterpret_cast<uintptr_t>(y_out) & 7))
         return EXL3_E_BAD_SHAPE;
-    const long long gy = ((long long)rows + BM - 1) / BM;
-    if (gy > 65535) return EXL3_E_BAD_SHAPE;
-    const dim3 grid((unsigned)(tn_count / 8), (unsigned)gy);
+    if (ldx * 2 * 256 >= (1ull << 31)) return EXL3_E_BAD_SHAPE;  // 32-bit row offsets inside a block
+    GemmPlan p = plan_gemm(rows, in_tiles, tn_count, workspace != nullptr);
+    const size_t need = (size_t)p.split_tiles * p.split * (32 * p.mi) * kGemmBN * sizeof(float);
+    if (need > workspace_bytes || (reinterpret_cast<uintptr_t>(workspace) & 15))
+        p = plan_gemm(rows, in_tiles, tn_count, false);
+    if ((long long)p.full_tiles + (long long)p.split_tiles * p.split > 0x7fffffffLL)
+        return EXL3_E_BAD_SHAPE;
+    float* partial = reinterpret_cast<float*>(workspace);
     return dispatch_k_cb(K, cb, [&](auto k, auto c) {
-        gemm_kernel<k.value, c.value><<<grid, dim3(256), 0, stream>>>(
-            reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<const half_t*>(xh),
-            reinterpret_cast<half_t*>(y_out), rows, ldx, ldy, in_tiles, out_tiles, tn_offset);
-        return launch_status();
+        if (p.mi == 2)
+            return launch_gemm_mi<k.value, c.value, 2>(p, xh, rows, ldx, trellis, in_tiles,
+                                                       out_tiles, tn_offset, tn_count, y_out, ldy,
+                                                       partial, stream);
+        return launch_gemm_mi<k.value, c.value, 8>(p, xh, rows, ldx, trellis, in_tiles, out_tiles,
+                                                   tn_offset, tn_count, y_out, ldy, partial,
+                                                   stream);
     });
 }
 
 }  // namespace exl3
 
+EXL3_EXPORT size_t exl3_gemm_workspace_bytes(int rows, int in_tiles, int tn_count) {
+    if (rows < 1 || in_tiles < 4 || tn_count < 8) return 0;
+    return exl3::gemm_workspace_bytes(rows, in_tiles, tn_count);
+}
+
 EXL3_EXPORT int exl3_gemm(const uint16_t* xh, int rows, size_t ldx, const uint16_t* trellis,
                           int in_tiles, int out_tiles, int K, int cb, int tn_offset, int tn_count,
-                          uint16_t* y_out, size_t ldy, void* stream) {
+                          uint16_t* y_out, size_t ldy, void* workspace, size_t workspace_bytes,
+                          void* stream) {
     return exl3::launch_gemm(xh, rows, ldx, trellis, in_tiles, out_tiles, K, cb, tn_offset,
-                             tn_count, y_out, ldy, exl3::as_stream(stream));
+                             tn_count, y_out, ldy, workspace, workspace_bytes,
+                             exl3::as_stream(stream));
 }

@@ -437,13 +437,6 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __res
 
 // Tuning knobs read once from the environment (the reference selects kernel
 // variants the same way, ponyexl3/mlx/gemv_metal.py:1017-1020).
-static int env_int(const char* name, int dflt, int lo, int hi) {
-    const char* v = getenv(name);
-    if (!v || !*v) return dflt;
-    const int x = atoi(v);
-    return x < lo ? lo : (x > hi ? hi : x);
-}
-
 GemvPlan plan_gemv(int rows, int in_tiles, int n_groups) {
     (void)rows;
     // Aim for kWavesPerSimd waves per SIMD over the 256*4 SIMDs, but never fewer

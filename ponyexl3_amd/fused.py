@@ -10,12 +10,10 @@ Hadamard block never straddles two members).
 
 from __future__ import annotations
 
-import ctypes
-
 import numpy as np
 import torch
 
-from . import _lib, ops
+from . import ops
 from .layer import EXL3Layer, codebook_mode_from_flags, unpack_signs_or_pass
 
 
@@ -82,18 +80,13 @@ class FusedEXL3Group(torch.nn.Module):
             xh = ops.had128_pre(x2d, self._suh_stack)  # (rows, n_sub, in)
             n_sub = len(self._out_features)
             yraw = torch.empty((rows, total_out), dtype=torch.float16, device=x2d.device)
-            lib = _lib.load()
-            in_tiles, out_tiles = self.in_features // 16, total_out // 16
             tn0 = 0
             for i, n in enumerate(self._out_features):
-                rc = lib.exl3_gemm(
-                    ctypes.c_void_p(xh.data_ptr() + 2 * i * self.in_features), rows,
-                    n_sub * self.in_features, ctypes.c_void_p(self._trellis.data_ptr()),
-                    in_tiles, out_tiles, self._k, self._cb, tn0, n // 16,
-                    ctypes.c_void_p(yraw.data_ptr() + 2 * 16 * tn0), total_out,
-                    ctypes.c_void_p(torch.cuda.current_stream().cuda_stream),
+                ops.gemm_into(
+                    xh.data_ptr() + 2 * i * self.in_features, rows, n_sub * self.in_features,
+                    self._trellis, self._k, self._cb, tn0, n // 16,
+                    yraw.data_ptr() + 2 * 16 * tn0, total_out, x2d.device,
                 )
-                _lib.check(rc, "exl3_gemm")
                 tn0 += n // 16
             y = ops.had128_post(yraw, self._svh_cat)
         outs = torch.split(y, self._out_features, dim=-1)

@@ -49,6 +49,22 @@ def workspace(device, nbytes: int) -> torch.Tensor:
     return buf
 
 
+_gemm_workspaces: dict = {}
+
+
+def gemm_workspace(device, nbytes: int):
+    """Per-device scratch for the prefill GEMM's fp32 partial tiles (kept apart
+    from ``workspace``, which holds the GEMM's operands during a layer forward)."""
+    if nbytes <= 0:
+        return None
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    buf = _gemm_workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
+        _gemm_workspaces[key] = buf
+    return buf
+
+
 _counters: dict = {}
 
 
@@ -299,12 +315,25 @@ def inner_gemm(xh, trellis, k: int, cb: int, tn_offset: int = 0, tn_count: int |
     if n_in % 64 or tn_count % 8 or tn_offset < 0 or tn_offset + tn_count > out_tiles:
         raise ValueError("prefill GEMM needs in % 64 == 0 and a 128-column aligned slice")
     y = torch.empty((rows, tn_count * 16), dtype=torch.float16, device=xh.device)
-    rc = _lib.load().exl3_gemm(
-        _ptr(xh), rows, n_in, _ptr(trellis), in_tiles, out_tiles, int(k), int(cb),
-        int(tn_offset), int(tn_count), _ptr(y), tn_count * 16, _stream(),
+    gemm_into(xh.data_ptr(), rows, n_in, trellis, k, cb, tn_offset, tn_count, y.data_ptr(),
+              tn_count * 16, xh.device)
+    return y
+
+
+def gemm_into(xh_ptr: int, rows: int, ldx: int, trellis, k: int, cb: int, tn_offset: int,
+              tn_count: int, y_ptr: int, ldy: int, device) -> None:
+    """``exl3_gemm`` on raw device addresses (strided activations / output slices),
+    with the split-tile scratch taken from the per-device GEMM workspace."""
+    lib = _lib.load()
+    in_tiles, out_tiles = _trellis_dims(trellis, k)
+    nbytes = lib.exl3_gemm_workspace_bytes(int(rows), in_tiles, int(tn_count))
+    ws = gemm_workspace(device, nbytes)
+    rc = lib.exl3_gemm(
+        ctypes.c_void_p(xh_ptr), int(rows), int(ldx), _ptr(trellis), in_tiles, out_tiles, int(k),
+        int(cb), int(tn_offset), int(tn_count), ctypes.c_void_p(y_ptr), int(ldy),
+        _ptr(ws) if ws is not None else None, int(nbytes), _stream(),
     )
     _lib.check(rc, "exl3_gemm")
-    return y
 
 
 def linear_forward(x2d, trellis, k, cb, suh=None, svh=None, bias=None, group_sub=None,

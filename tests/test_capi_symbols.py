@@ -58,7 +58,7 @@ def test_argument_errors_before_launch(lib):
     assert lib.exl3_had128_post(p, 0, 2, 0, 1, 128, None, None, p, None) == _lib.EXL3_E_BAD_SHAPE
     assert lib.exl3_gemv(p, 9, 1, p, 8, 8, 4, 0, None, None, 1, p, p, 1 << 20, None) == _lib.EXL3_E_BAD_SHAPE
     assert lib.exl3_gemv(p, 1, 2, p, 8, 8, 4, 0, None, None, 1, p, p, 1 << 20, None) == _lib.EXL3_E_BAD_INDEX
-    assert lib.exl3_gemm(p, 32, 100, p, 8, 8, 4, 0, 0, 8, p, 128, None) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_gemm(p, 32, 100, p, 8, 8, 4, 0, 0, 8, p, 128, None, 0, None) == _lib.EXL3_E_BAD_SHAPE
     assert lib.exl3_linear_forward(p, 1, p, 8, 8, 4, 0, None, 1, None, None, None, p, p, 16, None, 0, None) == _lib.EXL3_E_WORKSPACE
     assert lib.exl3_linear_forward(p, 1, p, 7, 8, 4, 0, None, 1, None, None, None, p, p, 1 << 20, None, 0, None) == _lib.EXL3_E_BAD_SHAPE
     assert lib.exl3_linear_forward(p, 1, p, 8, 16, 4, 0, None, 1, None, None, None, p, p, 1 << 20, p, 1, None) == _lib.EXL3_E_WORKSPACE

@@ -73,6 +73,60 @@ def test_config3_prefill_against_decoded_weights(cuda, oracle):
     assert float(err) < 5e-4
 
 
+@pytest.mark.parametrize("rows", [40, 300])
+def test_split_tiles_match_oracle_and_unsplit(cuda, oracle, rows):
+    """Few tiles and a deep reduction: every tile is cut into reduction ranges
+    whose fp32 partial tiles a second kernel adds. Checked against the oracle,
+    against the same call without a workspace (no split) and for run-to-run
+    determinism."""
+    import ctypes
+
+    from ponyexl3_amd import _lib, ops
+
+    rng = np.random.default_rng(43 + rows)
+    tr_np = rng.integers(0, 65536, size=(128, 64, 64), dtype=np.uint16)  # 2048 -> 1024, K = 4
+    tr = ops.as_trellis_tensor(tr_np, cuda)
+    xh_np = rng.standard_normal((rows, 2048)).astype(np.float16)
+    xh = _t(xh_np, cuda)
+    lib = _lib.load()
+    assert lib.exl3_gemm_workspace_bytes(rows, 128, 64) > 0  # this shape does split
+    print(f"gemm split rows={rows}", flush=True)
+    y1 = ops.inner_gemm(xh, tr, 4, 0)
+    y2 = ops.inner_gemm(xh, tr, 4, 0)
+    assert torch.equal(y1, y2)
+    ref = xh_np.astype(np.float64) @ oracle.decode_trellis(tr_np, 4, 0).astype(np.float64)
+    assert rel_l2(y1.cpu().numpy(), ref) < 5e-4
+    y0 = torch.empty_like(y1)
+    rc = lib.exl3_gemm(
+        ctypes.c_void_p(xh.data_ptr()), rows, 2048, ctypes.c_void_p(tr.data_ptr()), 128, 64, 4, 0,
+        0, 64, ctypes.c_void_p(y0.data_ptr()), 1024, None, 0,
+        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    assert rel_l2(y0.cpu().numpy(), ref) < 5e-4
+    assert rel_l2(y0.cpu().numpy(), y1.cpu().numpy()) < 5e-4
+
+
+@pytest.mark.parametrize("n_in,n_out", [(17408, 5120), (5120, 34816)])
+def test_config3_split_shapes_against_decoded_weights(cuda, n_in, n_out):
+    """M = 2048 on down_proj (160 tiles, all split three ways) and gate+up
+    (1088 tiles: four full rounds and 64 tiles split four ways) against the
+    bit-exact decoded weights times xh in fp32."""
+    from ponyexl3_amd import ops
+
+    g = torch.Generator().manual_seed(n_in)
+    tr = torch.randint(-32768, 32767, (n_in // 16, n_out // 16, 64), generator=g, dtype=torch.int16).to(cuda)
+    xh = (torch.randn((2048, n_in), generator=g) * 0.1).to(torch.float16).to(cuda)
+    print(f"gemm config3 {n_in}->{n_out}", flush=True)
+    y = ops.inner_gemm(xh, tr, 4, 0)
+    w = ops.decode_full(tr, 4, 0)
+    worst = 0.0
+    for c0 in range(0, n_out, 8192):  # fp32 reference in column slabs
+        ref = xh.float() @ w[:, c0:c0 + 8192].float()
+        err = (y[:, c0:c0 + 8192].float() - ref).norm() / ref.norm()
+        worst = max(worst, float(err))
+    assert worst < 5e-4
+
+
 def test_errors(cuda):
     from ponyexl3_amd import ops
 
