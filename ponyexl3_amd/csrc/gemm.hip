@@ -189,9 +189,6 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
         constexpr int s = decltype(slot)::value;
         const int stage = i & 1;
         const int k = k_begin + i;
-        load_a(clamp_k(k + 1), stage ^ 1);
-        const LaneWords<K> lw = finish_lane_words<K>(w_reg[s], lane);
-        load_w(clamp_k(k + 3), slot);
         const half_t* as = a_frag + stage * STAGE_A;
         const half_t* bs = b_frag + stage * STAGE_B;
         half_t* bdst = b_s + (stage ^ 1) * STAGE_B;
@@ -208,15 +205,24 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
         // MI groups per step, A fragments are requested two groups ahead.
         constexpr int G = MI;
         constexpr int GH = MI / 2;  // groups per 32-deep half
+        constexpr int EPG = 16 / G;  // decode elements per group
         auto lda_group = [&](auto gi_c) {
             constexpr int gi = decltype(gi_c)::value;
             af[gi % 3][0] = lda(gi / GH, 2 * (gi % GH));
             af[gi % 3][1] = lda(gi / GH, 2 * (gi % GH) + 1);
         };
+        // The first fragments are requested right after the barrier; the fills of the
+        // other stage and the first slice of decode work are issued while they fly.
 #pragma unroll
         for (int j = 0; j < 4; j++) bf[j] = ldb(0, j);
         lda_group(std::integral_constant<int, 0>{});
         lda_group(std::integral_constant<int, 1>{});
+        __builtin_amdgcn_sched_barrier(0);
+        load_a(clamp_k(k + 1), stage ^ 1);
+        const LaneWords<K> lw = finish_lane_words<K>(w_reg[s], lane);
+        __builtin_amdgcn_sched_barrier(0);  // keeps the trellis load behind the direct loads
+        load_w(clamp_k(k + 3), slot);
+        static_for<0, EPG>([&](auto e) { decode_element(lw, e, quad, bdst); });
         __builtin_amdgcn_sched_barrier(0);
         static_for<0, G>([&](auto gi_c) {
             constexpr int gi = decltype(gi_c)::value;
@@ -232,11 +238,15 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
 #pragma unroll
                 for (int j = 0; j < 4; j++) bf[j] = ldb(1, j);
             }
-            static_for<gi * (16 / G), (gi + 1) * (16 / G)>(
-                [&](auto e) { decode_element(lw, e, quad, bdst); });
+            if constexpr (gi + 1 < G)
+                static_for<(gi + 1) * EPG, (gi + 2) * EPG>(
+                    [&](auto e) { decode_element(lw, e, quad, bdst); });
             __builtin_amdgcn_sched_barrier(0);
         });
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the direct loads of stage^1 have landed
+        // Memory operations retire in order and at least one trellis load was issued
+        // after the direct loads of stage^1: with at most one load outstanding those
+        // have landed, and the trellis prefetch may stay in flight across the barrier.
+        asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
         __syncthreads();
     };
 
