@@ -178,7 +178,12 @@ def main():
         step(L)
     torch.cuda.synchronize()
 
+    # HIP graphs as a decoder would use them: one graph holds the steps of all
+    # n_layers layer copies back to back (a graph launch costs a few microseconds
+    # whatever it holds); single-layer graphs cover a step count that is not a
+    # multiple of n_layers.
     graphs = None
+    graph_all = None
     if not args.no_graph:
         try:
             graphs = []
@@ -187,23 +192,34 @@ def main():
                 with torch.cuda.graph(gr):
                     keep = step(L)
                 graphs.append((gr, keep))
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                keep = [step(L) for L in range(n_layers)]
+            graph_all = (gr, keep)
             torch.cuda.synchronize()
         except Exception as e:  # noqa: BLE001
             print(f"HIP graph capture failed ({e!r}); timing eager launches", file=sys.stderr)
             graphs = None
+            graph_all = None
 
-    def run(i):
-        if graphs is not None:
-            graphs[i % n_layers][0].replay()
-        else:
-            step(i % n_layers)
+    def run_steps(count):
+        """Exactly `count` layer steps, layer copies in rotation."""
+        i = 0
+        while i < count:
+            if graph_all is not None and i % n_layers == 0 and count - i >= n_layers:
+                graph_all[0].replay()
+                i += n_layers
+            elif graphs is not None:
+                graphs[i % n_layers][0].replay()
+                i += 1
+            else:
+                step(i % n_layers)
+                i += 1
 
-    for i in range(args.warmup):
-        run(i)
+    run_steps(args.warmup)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
-        run(i)
+    run_steps(args.steps)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
@@ -274,7 +290,8 @@ def main():
                         "one step = " + ", ".join(n for n, _, _ in LAYER) + " of one layer",
             "bytes_per_step": bytes_per_step,
             "weight_copies_rotated": n_layers,
-            "launch": "hip-graph replay" if graphs is not None else "eager",
+            "launch": (f"hip-graph replay, {n_layers} layer steps per graph" if graph_all is not None
+                       else "eager"),
         },
         "roofline": roofline,
     }
@@ -297,6 +314,23 @@ def _time_ms(fn, reps, warm=3):
         b.record()
     torch.cuda.synchronize()
     return float(np.mean([a.elapsed_time(b) for a, b in evs]))
+
+
+def _time_batch_ms(fn, reps, warm=10):
+    """Mean time of back-to-back calls (the queue never drains, so launch latency
+    of an idle device is not part of it)."""
+    import torch
+
+    for _ in range(warm):
+        fn()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps
 
 
 def bench_prefill(dev, layer, xs):
@@ -342,21 +376,49 @@ def bench_moe(dev):
             dn_trellis=rnd(H // 16, E * D // 16, 16 * K_BITS), dn_suh=sgn(E, H), dn_svh=sgn(E, D),
             k=K_BITS, cb=CB))
     res = {}
+    per_graph = 32  # chains per graph, each with its own routing, alternating weight copies
     for T in (1, 8):
         x = torch.from_numpy((rng.standard_normal((1, T, D)) * 0.25).astype(np.float16)).to(dev)
-        logits = torch.from_numpy(rng.standard_normal((T, E)).astype(np.float32)).to(dev)
-        inds, _ = route_topk(logits, kk)
-        distinct = int(torch.unique(inds).numel())
-        idx = inds.reshape(1, T, kk)
-        it = [0]
+        # Routing differs from chain to chain so that a replay streams far more expert
+        # weights than the 256 MB last-level cache holds: at one token the 32 chains
+        # of a graph use 32 disjoint top-8 sets (all 256 experts of both copies,
+        # 2 x 403 MB); at eight tokens every chain draws fresh router logits.
+        idxs, distinct = [], []
+        perm = rng.permutation(E)
+        for c in range(per_graph):
+            if T == 1:
+                inds = torch.from_numpy(perm[(c * kk) % E:(c * kk) % E + kk].astype(np.int32)).to(dev).reshape(1, kk)
+            else:
+                logits = torch.from_numpy(rng.standard_normal((T, E)).astype(np.float32)).to(dev)
+                inds, _ = route_topk(logits, kk)
+            distinct.append(int(torch.unique(inds).numel()))
+            idxs.append(inds.reshape(1, T, kk).to(torch.int32).contiguous())
+        for c in range(per_graph):  # warm-up outside any capture (workspaces, counters)
+            moes[c % copies](x, idxs[c])
+        torch.cuda.synchronize()
+        launch = "eager"
+        graph = None
+        try:  # device time of the chain: replay it from a HIP graph like the decode step
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                keep = [moes[c % copies](x, idxs[c]) for c in range(per_graph)]
+            graph = (gr, keep)
+            launch = f"hip-graph replay, {per_graph} chains per graph"
+        except Exception as e:  # noqa: BLE001
+            print(f"MoE graph capture failed ({e!r}); timing eager launches", file=sys.stderr)
 
         def fn():
-            moes[it[0] % copies](x, idx)
-            it[0] += 1
+            if graph is not None:
+                graph[0].replay()
+            else:
+                for c in range(per_graph):
+                    moes[c % copies](x, idxs[c])
 
-        ms = _time_ms(fn, reps=50)
-        nbytes = distinct * 3 * D * H * K_BITS // 8
-        res[f"tokens_{T}"] = {"us": round(ms * 1e3, 2), "distinct_experts": distinct,
+        ms = _time_batch_ms(fn, reps=20, warm=3) / per_graph
+        mean_distinct = float(np.mean(distinct))
+        nbytes = mean_distinct * 3 * D * H * K_BITS // 8
+        res[f"tokens_{T}"] = {"us": round(ms * 1e3, 2), "launch": launch,
+                              "distinct_experts": round(mean_distinct, 1),
                               "MB": round(nbytes / 1e6, 2), "GBps": round(nbytes / ms / 1e6, 1),
                               "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
     return {"moe": res}

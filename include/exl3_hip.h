@@ -197,13 +197,20 @@ size_t exl3_linear_workspace_bytes(int rows, int in_features, int out_features, 
  *   activation  0 = silu (SwiGLU), 1 = tanh-gelu (GeGLU) (ponyexl3/mlx/exl3_moe.py:62-75)
  *   y           fp16 [tokens][top_k][D]
  *   workspace   at least exl3_moe_workspace_bytes(tokens, top_k, D, H)
+ *   counters    NULL, or int32[counters_len] with counters_len >=
+ *               tokens*top_k*(H/128 + D/128), zero on entry and zero again on
+ *               exit. With counters the chain is two launches, the reference's
+ *               A2/B2 pair (ponyexl3/mlx/exl3_moe.py:345-422: gate/up, then
+ *               GLU + rotation + down); without, five launches that need no
+ *               state between calls. Calls that overlap on one counters array race.
  * Only the selected experts' trellis blocks are read.
  */
 int exl3_moe_forward(const uint16_t *x, int tokens, const int32_t *indices, int top_k,
                      const uint16_t *gu_trellis, const uint16_t *gu_suh, const uint16_t *gu_svh,
                      const uint16_t *dn_trellis, const uint16_t *dn_suh, const uint16_t *dn_svh,
                      int num_experts, int D, int H, int K, int cb, int activation, uint16_t *y,
-                     void *workspace, size_t workspace_bytes, void *stream);
+                     void *workspace, size_t workspace_bytes, int32_t *counters,
+                     size_t counters_len, void *stream);
 
 size_t exl3_moe_workspace_bytes(int tokens, int top_k, int D, int H);
 

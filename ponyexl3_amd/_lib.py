@@ -48,7 +48,8 @@ PROTOTYPES = {
     "exl3_linear_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "exl3_moe_forward": (
         _i,
-        [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _sz, _vp],
+        [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _sz, _vp,
+         _sz, _vp],
     ),
     "exl3_moe_workspace_bytes": (_sz, [_i, _i, _i, _i]),
 }

@@ -1,0 +1,142 @@
+// Shared pieces of the small-batch kernels (rows 1..8): the per-wave streaming
+// loop that rotates or stages a 128-wide block of activations in LDS and runs
+// the decode + dot pipeline over the block's 8 tile rows, and the 128-point
+// Walsh-Hadamard butterfly on two values per lane.
+#pragma once
+
+#include "exl3_device.hpp"
+
+namespace exl3 {
+
+constexpr float kHadScaleF = 0.088388347648318440550f;  // 1/sqrt(128)
+
+template <int K>
+__device__ __forceinline__ void load_lane_words_nt(const uint32_t* __restrict__ p,
+                                                   uint32_t (&own)[K]) {
+#pragma unroll
+    for (int i = 0; i < K; i++) own[i] = __builtin_nontemporal_load(p + i);
+}
+
+// Unnormalised WHT over 128 values held as (a, b) = elements (2*lane, 2*lane+1);
+// same butterfly order as ponyexl3/ref/hadamard.py:16-30 (stage h pairs i, i+h).
+__device__ __forceinline__ void wht128_lanes(float& a, float& b, int lane) {
+    const float s = a + b, d = a - b;
+    a = s;
+    b = d;
+#pragma unroll
+    for (int bit = 0; bit < 6; bit++) {
+        const int mask = 1 << bit;
+        const float pa = __shfl_xor(a, mask, kWave);
+        const float pb = __shfl_xor(b, mask, kWave);
+        const bool upper = (lane & mask) != 0;
+        a = upper ? pa - a : a + pa;
+        b = upper ? pb - b : b + pb;
+    }
+}
+
+// One wave streams tile rows [tk_begin, tk_end) (both multiples of 8, non-empty)
+// of the 8 tile columns that start at `base` (already offset by lane*K dwords)
+// and accumulates acc[m][0..1] += x[m][rows of the tile] . W[:, column u / u+8].
+//
+// Activations enter through the wave's own LDS slot xw[MT][128], one 128-wide
+// block (8 tile rows) at a time:
+//   ROTATE  xw = fp16(had128(x * suh) / sqrt(128))   (ponyexl3/ref/forward.py:32-34)
+//   else    xw = x                                   (x is already rotated)
+// The raw block after the current one is in flight while the current one is
+// used; a tile row's 16 activations come back with two broadcast ds_read_b128.
+// kSlots wave-wide trellis loads are kept in flight.
+template <int K, int CB, int MT, bool ROTATE>
+__device__ __forceinline__ void stream_block_rows(const uint32_t* __restrict__ base,
+                                                  size_t row_words, int tk_begin, int tk_end,
+                                                  const half_t* __restrict__ x, size_t x_stride,
+                                                  int rows, const half_t* __restrict__ suh_row,
+                                                  half_t (*xw)[128], int lane,
+                                                  float (&acc)[MT][2]) {
+    half2_t xraw[MT], sraw;
+    auto fetch_block = [&](int blk) {
+        const int off = blk * 128 + 2 * lane;
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            const int r = m < rows ? m : 0;
+            xraw[m] = *reinterpret_cast<const half2_t*>(x + (size_t)r * x_stride + off);
+        }
+        if (ROTATE && suh_row) sraw = *reinterpret_cast<const half2_t*>(suh_row + off);
+    };
+    auto stage_block = [&]() {
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            half2_t o = xraw[m];
+            if constexpr (ROTATE) {
+                float a = (float)xraw[m].x, b = (float)xraw[m].y;
+                if (suh_row) {
+                    a = __fmul_rn(a, (float)sraw.x);
+                    b = __fmul_rn(b, (float)sraw.y);
+                }
+                wht128_lanes(a, b, lane);
+                o.x = (half_t)__fmul_rn(a, kHadScaleF);
+                o.y = (half_t)__fmul_rn(b, kHadScaleF);
+            }
+            *reinterpret_cast<half2_t*>(&xw[m][2 * lane]) = o;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+    struct XTile {
+        uint4_t q[MT][2];
+    };
+    auto load_x = [&](int row_in_block) {
+        XTile t;
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            const uint4_t* xp = reinterpret_cast<const uint4_t*>(&xw[m][row_in_block * 16]);
+            t.q[m][0] = xp[0];
+            t.q[m][1] = xp[1];
+        }
+        return t;
+    };
+    auto consume = [&](const uint32_t (&words)[K], uint32_t prev, const XTile& xt) {
+        const LaneWords<K> lw = make_lane_words<K>(prev, words);
+        half2_t wp[16];
+        decode_lane<K, CB>(lw, wp);
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            const uint4_t x0 = xt.q[m][0], x1 = xt.q[m][1];
+            const half2_t xv[8] = {bits_to_half2(x0.x), bits_to_half2(x0.y), bits_to_half2(x0.z),
+                                   bits_to_half2(x0.w), bits_to_half2(x1.x), bits_to_half2(x1.y),
+                                   bits_to_half2(x1.z), bits_to_half2(x1.w)};
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                acc[m][0] = dot2(wp[j], xv[j], acc[m][0]);
+                acc[m][1] = dot2(wp[8 + j], xv[j], acc[m][1]);
+            }
+        }
+    };
+    // Ranges are whole blocks, so the staging sits outside the unrolled 8-step
+    // pipeline and the LDS offsets of the activations are compile-time constants.
+    constexpr int kSlots = 4;  // wave-wide loads in flight (divides the 8 steps of a block)
+    uint32_t buf[kSlots][K];
+#pragma unroll
+    for (int s = 0; s < kSlots; s++)
+        load_lane_words_nt<K>(base + (size_t)min(tk_begin + s, tk_end - 1) * row_words, buf[s]);
+    fetch_block(tk_begin >> 3);
+    uint32_t prev = neighbour_word(buf[0][K - 1], lane);
+    for (int tkb = tk_begin; tkb < tk_end; tkb += 8) {
+        stage_block();
+        if (tkb + 8 < tk_end) fetch_block((tkb >> 3) + 1);
+#pragma unroll
+        for (int s8 = 0; s8 < 8; s8++) {
+            const int tk = tkb + s8;
+            const int slot = s8 & (kSlots - 1);
+            const uint32_t prev_next = neighbour_word(buf[(slot + 1) & (kSlots - 1)][K - 1], lane);
+            const XTile xt = load_x(s8);
+            __builtin_amdgcn_sched_barrier(0);
+            consume(buf[slot], prev, xt);
+            const int tn = min(tk + kSlots, tk_end - 1);
+            load_lane_words_nt<K>(base + (size_t)tn * row_words, buf[slot]);
+            __builtin_amdgcn_sched_barrier(0);
+            prev = prev_next;
+        }
+    }
+}
+
+}  // namespace exl3

@@ -25,19 +25,13 @@
 // inner_gem_fused_mlx (ponyexl3/mlx/gemv_metal.py:109-232, 460-627, 1481-1515).
 #include "exl3_device.hpp"
 #include "exl3_host.hpp"
+#include "exl3_small.hpp"
 
 #include <stdlib.h>
 
 namespace exl3 {
 
 constexpr int kPrefetch = 6;  // wave-wide loads in flight per wave
-
-template <int K>
-__device__ __forceinline__ void load_lane_words_nt(const uint32_t* __restrict__ p,
-                                                   uint32_t (&own)[K]) {
-#pragma unroll
-    for (int i = 0; i < K; i++) own[i] = __builtin_nontemporal_load(p + i);
-}
 
 template <int K, int CB, int MT>
 __global__ __launch_bounds__(256) void gemv_kernel(
@@ -190,23 +184,6 @@ __global__ __launch_bounds__(256) void gemv_kernel(
 //     ever waits for another one, and the sum order is fixed, so the result is
 //     deterministic.
 // Counters must be zero on entry; they are zero again when the kernel ends.
-constexpr float kHadScaleF = 0.088388347648318440550f;  // 1/sqrt(128)
-
-__device__ __forceinline__ void wht128_lanes(float& a, float& b, int lane) {
-    const float s = a + b, d = a - b;
-    a = s;
-    b = d;
-#pragma unroll
-    for (int bit = 0; bit < 6; bit++) {
-        const int mask = 1 << bit;
-        const float pa = __shfl_xor(a, mask, kWave);
-        const float pb = __shfl_xor(b, mask, kWave);
-        const bool upper = (lane & mask) != 0;
-        a = upper ? pa - a : a + pa;
-        b = upper ? pb - b : b + pb;
-    }
-}
-
 template <int K, int CB, int MT>
 __global__ __launch_bounds__(256) void linear_small_kernel(
     const uint32_t* __restrict__ trellis, const half_t* __restrict__ x,
@@ -232,98 +209,11 @@ __global__ __launch_bounds__(256) void linear_small_kernel(
 #pragma unroll
     for (int m = 0; m < MT; m++) acc[m][0] = acc[m][1] = 0.f;
 
-    // ---- input Hadamard, one 128-block (8 tile rows) at a time
-    half2_t xraw[MT], sraw;
-    auto fetch_block = [&](int blk) {
-        const int off = blk * 128 + 2 * lane;
-#pragma unroll
-        for (int m = 0; m < MT; m++) {
-            const int r = m < rows ? m : 0;
-            xraw[m] = *reinterpret_cast<const half2_t*>(x + (size_t)r * in_features + off);
-        }
-        if (suh_row) sraw = *reinterpret_cast<const half2_t*>(suh_row + off);
-    };
-    auto rotate_block = [&]() {
-#pragma unroll
-        for (int m = 0; m < MT; m++) {
-            float a = (float)xraw[m].x, b = (float)xraw[m].y;
-            if (suh_row) {
-                a = __fmul_rn(a, (float)sraw.x);
-                b = __fmul_rn(b, (float)sraw.y);
-            }
-            wht128_lanes(a, b, lane);
-            half2_t o;
-            o.x = (half_t)__fmul_rn(a, kHadScaleF);
-            o.y = (half_t)__fmul_rn(b, kHadScaleF);
-            *reinterpret_cast<half2_t*>(&xs[wave][m][2 * lane]) = o;
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-    };
-
-    // One pipeline step (see gemv_kernel): neighbour dword of the next slot and
-    // the 16 activations of this tile row (two broadcast LDS reads) are requested
-    // first, then the slot is decoded, multiplied and refilled.
-    struct XTile {
-        uint4_t q[MT][2];
-    };
-    auto load_x = [&](int row_in_block) {
-        XTile t;
-#pragma unroll
-        for (int m = 0; m < MT; m++) {
-            const uint4_t* xp = reinterpret_cast<const uint4_t*>(&xs[wave][m][row_in_block * 16]);
-            t.q[m][0] = xp[0];
-            t.q[m][1] = xp[1];
-        }
-        return t;
-    };
-    auto consume = [&](const uint32_t (&words)[K], uint32_t prev, const XTile& xt) {
-        const LaneWords<K> lw = make_lane_words<K>(prev, words);
-        half2_t wp[16];
-        decode_lane<K, CB>(lw, wp);
-#pragma unroll
-        for (int m = 0; m < MT; m++) {
-            const uint4_t x0 = xt.q[m][0], x1 = xt.q[m][1];
-            const half2_t xv[8] = {bits_to_half2(x0.x), bits_to_half2(x0.y), bits_to_half2(x0.z),
-                                   bits_to_half2(x0.w), bits_to_half2(x1.x), bits_to_half2(x1.y),
-                                   bits_to_half2(x1.z), bits_to_half2(x1.w)};
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                acc[m][0] = dot2(wp[j], xv[j], acc[m][0]);
-                acc[m][1] = dot2(wp[8 + j], xv[j], acc[m][1]);
-            }
-        }
-    };
-    // Splits are whole Hadamard blocks (8 tile rows), so the block rotation sits
-    // outside the unrolled 8-step pipeline and the LDS offsets of the activations
-    // are compile-time constants.
-    constexpr int kSlots = 4;  // wave-wide loads in flight (divides the 8 steps of a block)
-    if (active) {
-        uint32_t buf[kSlots][K];
-#pragma unroll
-        for (int s = 0; s < kSlots; s++)
-            load_lane_words_nt<K>(base + (size_t)min(tk_begin + s, tk_end - 1) * row_words, buf[s]);
-        fetch_block(tk_begin >> 3);
-        uint32_t prev = neighbour_word(buf[0][K - 1], lane);
-        for (int tkb = tk_begin; tkb < tk_end; tkb += 8) {
-            rotate_block();
-            if (tkb + 8 < tk_end) fetch_block((tkb >> 3) + 1);
-#pragma unroll
-            for (int s8 = 0; s8 < 8; s8++) {
-                const int tk = tkb + s8;
-                const int slot = s8 & (kSlots - 1);
-                const uint32_t prev_next =
-                    neighbour_word(buf[(slot + 1) & (kSlots - 1)][K - 1], lane);
-                const XTile xt = load_x(s8);
-                __builtin_amdgcn_sched_barrier(0);
-                consume(buf[slot], prev, xt);
-                const int tn = min(tk + kSlots, tk_end - 1);
-                load_lane_words_nt<K>(base + (size_t)tn * row_words, buf[slot]);
-                __builtin_amdgcn_sched_barrier(0);
-                prev = prev_next;
-            }
-        }
-    }
+    // ---- input Hadamard + decode/dot pipeline over this wave's blocks
+    if (active)
+        stream_block_rows<K, CB, MT, true>(base, row_words, tk_begin, tk_end, x,
+                                           (size_t)in_features, rows, suh_row, xs[wave], lane,
+                                           acc);
 
     // ---- the four waves of the workgroup are summed through LDS in wave order,
     // the workgroup stores ONE fp32 partial row, and the last workgroup of the

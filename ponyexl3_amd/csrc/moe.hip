@@ -4,7 +4,17 @@
 // stacked trellises are read: the GEMV kernel is pointed at them through
 // per-group tables built on the device from the routing indices.
 //
-// Launch chain (all on one stream):
+// Two launches when the caller provides zeroed counters:
+//   A. moe_gateup_kernel    per (slot, gate|up, 128 columns of H): input rotation
+//                           in the wave, decode GEMV over D, workgroup sum; the
+//                           last workgroup of a (slot, column block) adds the
+//                           partial rows of gate and up, applies post-Hadamard,
+//                           svh and the GLU and rotates the block for the down
+//                           projection (a Hadamard block of H is exactly one
+//                           128-column group of gate/up)
+//   B. moe_down_kernel      per (slot, 128 columns of D): decode GEMV over H on
+//                           the rotated block, sum, post-Hadamard, svh
+// Without counters the same result comes from a chain of five launches:
 //   1. moe_prep_kernel      rotated activations per (slot, proj) + group tables
 //   2. gemv_kernel          gate/up partial sums, fp32
 //   3. moe_glu_kernel       split reduction, post-Hadamard, svh, GLU, then the
@@ -17,27 +27,13 @@
 // (ponyexl3/mlx/exl3_moe.py:345-422) are what this replaces.
 #include "exl3_device.hpp"
 #include "exl3_host.hpp"
+#include "exl3_small.hpp"
+
+#include <algorithm>
 
 #pragma clang fp contract(off)
 
 namespace exl3 {
-
-constexpr float kHadScaleMoe = 0.088388347648318440550f;
-
-__device__ __forceinline__ void wht128_moe(float& a, float& b, int lane) {
-    const float s = a + b, d = a - b;
-    a = s;
-    b = d;
-#pragma unroll
-    for (int bit = 0; bit < 6; bit++) {
-        const int mask = 1 << bit;
-        const float pa = __shfl_xor(a, mask, kWave);
-        const float pb = __shfl_xor(b, mask, kWave);
-        const bool upper = (lane & mask) != 0;
-        a = upper ? pa - a : a + pa;
-        b = upper ? pb - b : b + pb;
-    }
-}
 
 // Routing indices come from the caller's device memory; an out-of-range value is
 // clamped so that it can never turn into an out-of-bounds read.
@@ -76,10 +72,10 @@ __global__ __launch_bounds__(256) void moe_prep_kernel(
     const half2_t sv = *reinterpret_cast<const half2_t*>(gu_suh + ((size_t)e * 2 + p) * D +
                                                          blk * 128 + 2 * lane);
     float a = (float)xv.x * (float)sv.x, b = (float)xv.y * (float)sv.y;
-    wht128_moe(a, b, lane);
+    wht128_lanes(a, b, lane);
     half2_t o;
-    o.x = (half_t)(a * kHadScaleMoe);
-    o.y = (half_t)(b * kHadScaleMoe);
+    o.x = (half_t)(a * kHadScaleF);
+    o.y = (half_t)(b * kHadScaleF);
     *reinterpret_cast<half2_t*>(xh_gu + (size_t)sp * D + blk * 128 + 2 * lane) = o;
 }
 
@@ -116,21 +112,21 @@ __global__ __launch_bounds__(256) void moe_glu_kernel(
             acc.y = acc.y + q.y;
         }
         float a = (float)(half_t)acc.x, b = (float)(half_t)acc.y;
-        wht128_moe(a, b, lane);
+        wht128_lanes(a, b, lane);
         const half2_t sv = *reinterpret_cast<const half2_t*>(gu_svh + (size_t)e * 2 * H + p * H +
                                                              blk * 128 + 2 * lane);
-        v[p][0] = (float)(half_t)(a * kHadScaleMoe * (float)sv.x);
-        v[p][1] = (float)(half_t)(b * kHadScaleMoe * (float)sv.y);
+        v[p][0] = (float)(half_t)(a * kHadScaleF * (float)sv.x);
+        v[p][1] = (float)(half_t)(b * kHadScaleF * (float)sv.y);
     }
     const float h0 = (float)(half_t)glu_act(v[0][0], v[1][0], activation);
     const float h1 = (float)(half_t)glu_act(v[0][1], v[1][1], activation);
     const half2_t ds =
         *reinterpret_cast<const half2_t*>(dn_suh + (size_t)e * H + blk * 128 + 2 * lane);
     float a = h0 * (float)ds.x, b = h1 * (float)ds.y;
-    wht128_moe(a, b, lane);
+    wht128_lanes(a, b, lane);
     half2_t o;
-    o.x = (half_t)(a * kHadScaleMoe);
-    o.y = (half_t)(b * kHadScaleMoe);
+    o.x = (half_t)(a * kHadScaleF);
+    o.y = (half_t)(b * kHadScaleF);
     *reinterpret_cast<half2_t*>(xh_dn + (size_t)s * H + blk * 128 + 2 * lane) = o;
 }
 
@@ -152,13 +148,190 @@ __global__ __launch_bounds__(256) void moe_finish_kernel(
         acc.y = acc.y + q.y;
     }
     float a = (float)(half_t)acc.x, b = (float)(half_t)acc.y;
-    wht128_moe(a, b, lane);
+    wht128_lanes(a, b, lane);
     const half2_t sv =
         *reinterpret_cast<const half2_t*>(dn_svh + (size_t)e * D + blk * 128 + 2 * lane);
     half2_t o;
-    o.x = (half_t)(a * kHadScaleMoe * (float)sv.x);
-    o.y = (half_t)(b * kHadScaleMoe * (float)sv.y);
+    o.x = (half_t)(a * kHadScaleF * (float)sv.x);
+    o.y = (half_t)(b * kHadScaleF * (float)sv.y);
     *reinterpret_cast<half2_t*>(y + off) = o;
+}
+
+
+// ---------------------------------------------------------------------------
+// Fused chain: shared tail of both kernels. The four waves of a workgroup are
+// added through LDS in wave order; returns the two sums of this lane's columns
+// (2*lane, 2*lane+1) to wave 0.
+__device__ __forceinline__ float2_t moe_wg_sum(float (*red)[128], const float (&acc)[1][2],
+                                               int lane, int wave) {
+    const int c0 = (lane >> 3) * 16 + (lane & 7);
+    red[wave][c0] = acc[0][0];
+    red[wave][c0 + 8] = acc[0][1];
+    __syncthreads();
+    float2_t v;
+    v.x = ((red[0][2 * lane] + red[1][2 * lane]) + red[2][2 * lane]) + red[3][2 * lane];
+    v.y = ((red[0][2 * lane + 1] + red[1][2 * lane + 1]) + red[2][2 * lane + 1]) +
+          red[3][2 * lane + 1];
+    return v;
+}
+
+// Partial rows cross workgroups through device-scope accesses only (the XCDs'
+// L2 caches are not coherent with each other): store, wait, bump the counter;
+// the workgroup that sees `expected - 1` is the last one and reads them back.
+__device__ __forceinline__ bool moe_publish(float* row, float2_t v, int* counter, int expected,
+                                            int lane) {
+    __hip_atomic_store(reinterpret_cast<uint64_t*>(row + 2 * lane),
+                       __builtin_bit_cast(uint64_t, v), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    int seen = 0;
+    if (lane == 0)
+        seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return __shfl(seen, 0, kWave) == expected - 1;
+}
+
+__device__ __forceinline__ float2_t moe_sum_rows(const float* rows, int n, int lane) {
+    float a = 0.f, b = 0.f;
+    for (int i = 0; i < n; i++) {
+        const float2_t f = __builtin_bit_cast(
+            float2_t, __hip_atomic_load(reinterpret_cast<const uint64_t*>(rows + i * 128 + 2 * lane),
+                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        a = __fadd_rn(a, f.x);
+        b = __fadd_rn(b, f.y);
+    }
+    return float2_t{a, b};
+}
+
+// fp16(had128(fp16(sum)) / sqrt(128) * sv): the finish of one EXL3 linear on one
+// 128-column block (ponyexl3/ref/forward.py:41-42).
+__device__ __forceinline__ void moe_finish_block(float2_t sum, half2_t sv, int lane, float& o0,
+                                                 float& o1) {
+    float a = (float)(half_t)sum.x, b = (float)(half_t)sum.y;
+    wht128_lanes(a, b, lane);
+    o0 = (float)(half_t)(a * kHadScaleF * (float)sv.x);
+    o1 = (float)(half_t)(b * kHadScaleF * (float)sv.y);
+}
+
+// grid = (slots * 2 * H/128, ceil((D/128) / 4)); wave w of workgroup (gid, q) owns
+// the Hadamard block 4q + w of D for slot s = gid / (2*hblocks), projection
+// p = (gid / hblocks) & 1 and column block hg = gid % hblocks.
+// part: fp32 [gid][n_wg][128]; counters[s*hblocks + hg] count 2*n_wg workgroups.
+template <int K, int CB>
+__global__ __launch_bounds__(256) void moe_gateup_kernel(
+    const uint32_t* __restrict__ gu_trellis, const half_t* __restrict__ x,
+    const int* __restrict__ indices, const half_t* __restrict__ gu_suh,
+    const half_t* __restrict__ gu_svh, const half_t* __restrict__ dn_suh, half_t* xh_dn,
+    float* part, int* counters, int top_k, int E, int D, int H, int activation) {
+    __shared__ __attribute__((aligned(16))) half_t xs[4][1][128];
+    __shared__ float red[4][128];
+    __shared__ float up_val[128];
+    __shared__ int last_flag;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int dblocks = D >> 7, hblocks = H >> 7;
+    const int n_wg = gridDim.y;
+    const int gid = blockIdx.x;
+    const int hg = gid % hblocks, sp = gid / hblocks;
+    const int s = sp >> 1, p = sp & 1;
+    const int e = clamp_expert(indices[s], E);
+    const int blk = blockIdx.y * 4 + wave;
+    float acc[1][2] = {{0.f, 0.f}};
+    if (blk < dblocks) {
+        const size_t row_words = (size_t)E * 2 * (H >> 4) * (8 * K);
+        const uint32_t* base =
+            gu_trellis + ((size_t)(p * E + e) * (H >> 4) + 8 * hg) * (8 * K) + lane * K;
+        stream_block_rows<K, CB, 1, true>(base, row_words, blk * 8, blk * 8 + 8,
+                                          x + (size_t)(s / top_k) * D, (size_t)D, 1,
+                                          gu_suh + ((size_t)e * 2 + p) * D, xs[wave], lane, acc);
+    }
+    const float2_t v = moe_wg_sum(red, acc, lane, wave);
+    int* counter = counters + s * hblocks + hg;
+    if (wave == 0) {
+        const bool last = moe_publish(part + ((size_t)gid * n_wg + blockIdx.y) * 128, v, counter,
+                                      2 * n_wg, lane);
+        if (lane == 0) last_flag = last;
+    }
+    __syncthreads();
+    if (!last_flag) return;
+    asm volatile("" ::: "memory");
+    // waves 0 and 1 finish gate and up, wave 0 then applies the GLU and rotates
+    float f0 = 0.f, f1 = 0.f;
+    if (wave < 2) {
+        const int gid_p = (s * 2 + wave) * hblocks + hg;
+        const float2_t sum = moe_sum_rows(part + (size_t)gid_p * n_wg * 128, n_wg, lane);
+        const half2_t sv = *reinterpret_cast<const half2_t*>(
+            gu_svh + (size_t)e * 2 * H + wave * H + hg * 128 + 2 * lane);
+        moe_finish_block(sum, sv, lane, f0, f1);
+        if (wave == 1) {
+            up_val[2 * lane] = f0;
+            up_val[2 * lane + 1] = f1;
+        }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    const float h0 = (float)(half_t)glu_act(f0, up_val[2 * lane], activation);
+    const float h1 = (float)(half_t)glu_act(f1, up_val[2 * lane + 1], activation);
+    const half2_t ds =
+        *reinterpret_cast<const half2_t*>(dn_suh + (size_t)e * H + hg * 128 + 2 * lane);
+    float a = h0 * (float)ds.x, b = h1 * (float)ds.y;
+    wht128_lanes(a, b, lane);
+    half2_t o;
+    o.x = (half_t)(a * kHadScaleF);
+    o.y = (half_t)(b * kHadScaleF);
+    *reinterpret_cast<half2_t*>(xh_dn + (size_t)s * H + hg * 128 + 2 * lane) = o;
+    if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// grid = (slots * D/128, ceil((H/128) / 4)); slot s = gid / dblocks, column block
+// og = gid % dblocks. xh_dn is already rotated. part: fp32 [gid][n_wg][128].
+template <int K, int CB>
+__global__ __launch_bounds__(256) void moe_down_kernel(
+    const uint32_t* __restrict__ dn_trellis, const half_t* __restrict__ xh_dn,
+    const int* __restrict__ indices, const half_t* __restrict__ dn_svh, half_t* __restrict__ y,
+    float* part, int* counters, int E, int D, int H) {
+    __shared__ __attribute__((aligned(16))) half_t xs[4][1][128];
+    __shared__ float red[4][128];
+    __shared__ int last_flag;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int dblocks = D >> 7, hblocks = H >> 7;
+    const int n_wg = gridDim.y;
+    const int gid = blockIdx.x;
+    const int og = gid % dblocks, s = gid / dblocks;
+    const int e = clamp_expert(indices[s], E);
+    const int blk = blockIdx.y * 4 + wave;
+    float acc[1][2] = {{0.f, 0.f}};
+    if (blk < hblocks) {
+        const size_t row_words = (size_t)E * (D >> 4) * (8 * K);
+        const uint32_t* base = dn_trellis + ((size_t)e * (D >> 4) + 8 * og) * (8 * K) + lane * K;
+        stream_block_rows<K, CB, 1, false>(base, row_words, blk * 8, blk * 8 + 8,
+                                           xh_dn + (size_t)s * H, (size_t)H, 1, nullptr, xs[wave],
+                                           lane, acc);
+    }
+    float2_t v = moe_wg_sum(red, acc, lane, wave);
+    if (n_wg > 1) {
+        int* counter = counters + gid;
+        if (wave == 0) {
+            const bool last = moe_publish(part + ((size_t)gid * n_wg + blockIdx.y) * 128, v,
+                                          counter, n_wg, lane);
+            if (lane == 0) last_flag = last;
+        }
+        __syncthreads();
+        if (!last_flag || wave != 0) return;
+        asm volatile("" ::: "memory");
+        v = moe_sum_rows(part + (size_t)gid * n_wg * 128, n_wg, lane);
+        if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else if (wave != 0) {
+        return;
+    }
+    const half2_t sv =
+        *reinterpret_cast<const half2_t*>(dn_svh + (size_t)e * D + og * 128 + 2 * lane);
+    float o0, o1;
+    moe_finish_block(v, sv, lane, o0, o1);
+    half2_t o;
+    o.x = (half_t)o0;
+    o.y = (half_t)o1;
+    *reinterpret_cast<half2_t*>(y + (size_t)s * D + og * 128 + 2 * lane) = o;
 }
 
 struct MoeWorkspace {
@@ -178,8 +351,12 @@ static MoeWorkspace moe_workspace(int tokens, int top_k, int D, int H) {
     w.xh_gu = align_up((size_t)slots * 2 * D * 2, 256);
     w.xh_dn = align_up((size_t)slots * H * 2, 256);
     w.tables = align_up((size_t)2 * (w.g_gu + w.g_dn) * sizeof(int), 256);
-    w.part_gu = align_up((size_t)w.plan_gu.n_partials() * w.g_gu * 128 * sizeof(float), 256);
-    w.part_dn = align_up((size_t)w.plan_dn.n_partials() * w.g_dn * 128 * sizeof(float), 256);
+    // partial rows per group: the chain's split plan or the fused kernels' one row per
+    // workgroup of four Hadamard blocks, whichever is larger
+    const int rows_gu = std::max(w.plan_gu.n_partials(), (D / 128 + 3) / 4);
+    const int rows_dn = std::max(w.plan_dn.n_partials(), (H / 128 + 3) / 4);
+    w.part_gu = align_up((size_t)rows_gu * w.g_gu * 128 * sizeof(float), 256);
+    w.part_dn = align_up((size_t)rows_dn * w.g_dn * 128 * sizeof(float), 256);
     w.o_xh_gu = 0;
     w.o_xh_dn = w.o_xh_gu + w.xh_gu;
     w.o_tables = w.o_xh_dn + w.xh_dn;
@@ -201,7 +378,8 @@ EXL3_EXPORT int exl3_moe_forward(const uint16_t* x, int tokens, const int32_t* i
                                  const uint16_t* gu_svh, const uint16_t* dn_trellis,
                                  const uint16_t* dn_suh, const uint16_t* dn_svh, int num_experts,
                                  int D, int H, int K, int cb, int activation, uint16_t* y,
-                                 void* workspace, size_t workspace_bytes, void* stream) {
+                                 void* workspace, size_t workspace_bytes, int32_t* counters,
+                                 size_t counters_len, void* stream) {
     using namespace exl3;
     if (int rc = check_k_cb(K, cb)) return rc;
     if (!x || !indices || !gu_trellis || !gu_suh || !gu_svh || !dn_trellis || !dn_suh || !dn_svh ||
@@ -224,6 +402,29 @@ EXL3_EXPORT int exl3_moe_forward(const uint16_t* x, int tokens, const int32_t* i
     float* part_gu = reinterpret_cast<float*>(base + w.o_part_gu);
     float* part_dn = reinterpret_cast<float*>(base + w.o_part_dn);
     const int slots = tokens * top_k;
+
+    if (counters) {
+        // two launches: gate/up + GLU + rotation, then down
+        const int hblocks = H / 128, dblocks = D / 128;
+        if (counters_len < (size_t)slots * (hblocks + dblocks)) return EXL3_E_WORKSPACE;
+        return dispatch_k_cb(K, cb, [&](auto k, auto c) {
+            moe_gateup_kernel<k.value, c.value>
+                <<<dim3((unsigned)(slots * 2 * hblocks), (unsigned)((dblocks + 3) / 4)), dim3(256),
+                   0, s>>>(reinterpret_cast<const uint32_t*>(gu_trellis),
+                           reinterpret_cast<const half_t*>(x), indices,
+                           reinterpret_cast<const half_t*>(gu_suh),
+                           reinterpret_cast<const half_t*>(gu_svh),
+                           reinterpret_cast<const half_t*>(dn_suh), xh_dn, part_gu, counters,
+                           top_k, num_experts, D, H, activation);
+            if (int rc = launch_status()) return rc;
+            moe_down_kernel<k.value, c.value>
+                <<<dim3((unsigned)(slots * dblocks), (unsigned)((hblocks + 3) / 4)), dim3(256), 0,
+                   s>>>(reinterpret_cast<const uint32_t*>(dn_trellis), xh_dn, indices,
+                        reinterpret_cast<const half_t*>(dn_svh), reinterpret_cast<half_t*>(y),
+                        part_dn, counters + (size_t)slots * hblocks, num_experts, D, H);
+            return launch_status();
+        });
+    }
 
     {
         const int waves = slots * 2 * (D / 128);

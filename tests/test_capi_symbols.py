@@ -62,8 +62,8 @@ def test_argument_errors_before_launch(lib):
     assert lib.exl3_linear_forward(p, 1, p, 8, 8, 4, 0, None, 1, None, None, None, p, p, 16, None, 0, None) == _lib.EXL3_E_WORKSPACE
     assert lib.exl3_linear_forward(p, 1, p, 7, 8, 4, 0, None, 1, None, None, None, p, p, 1 << 20, None, 0, None) == _lib.EXL3_E_BAD_SHAPE
     assert lib.exl3_linear_forward(p, 1, p, 8, 16, 4, 0, None, 1, None, None, None, p, p, 1 << 20, p, 1, None) == _lib.EXL3_E_WORKSPACE
-    assert lib.exl3_moe_forward(p, 1, p, 8, p, p, p, p, p, p, 4, 256, 100, 4, 0, 0, p, p, 1 << 20, None) == _lib.EXL3_E_BAD_SHAPE
-    assert lib.exl3_moe_forward(p, 1, p, 8, p, p, p, p, p, p, 4, 256, 128, 4, 0, 7, p, p, 1 << 20, None) == _lib.EXL3_E_UNSUPPORTED
+    assert lib.exl3_moe_forward(p, 1, p, 8, p, p, p, p, p, p, 4, 256, 100, 4, 0, 0, p, p, 1 << 20, None, 0, None) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_moe_forward(p, 1, p, 8, p, p, p, p, p, p, 4, 256, 128, 4, 0, 7, p, p, 1 << 20, None, 0, None) == _lib.EXL3_E_UNSUPPORTED
 
 
 def test_workspace_sizes(lib):

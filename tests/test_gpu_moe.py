@@ -45,6 +45,34 @@ def test_moe_matches_oracle(cuda, oracle, tokens, k, mcg, act):
     assert rel_l2(y[0], ref) <= TOL
 
 
+@pytest.mark.parametrize("tokens", [1, 8])
+def test_two_launch_and_five_launch_chains(cuda, oracle, tokens):
+    """D and H of five Hadamard blocks each: both kernels of the two-launch chain
+    run two workgroups per column block (one of them with a single active wave)
+    and meet through the counters. Checked against the oracle, against the
+    five-launch chain, and twice in a row (the counters must be left at zero)."""
+    from ponyexl3_amd import EXL3SwitchGLU, ops
+
+    E, D, H, kk, k = 5, 640, 640, 2, 4
+    gate, up, down = _experts(E, D, H, k, False, 700)
+    moe = EXL3SwitchGLU.from_layers(gate, up, down)
+    rng = np.random.default_rng(70 + tokens)
+    x = (rng.standard_normal((tokens, D)) * 0.5).astype(np.float16)
+    idx = np.stack([rng.permutation(E)[:kk] for _ in range(tokens)]).astype(np.int32)
+    xt, it = torch.from_numpy(x).to(cuda), torch.from_numpy(idx).to(cuda)
+    args = (xt, it, moe._gu_trellis, moe._gu_suh, moe._gu_svh, moe._dn_trellis, moe._dn_suh, moe._dn_svh,
+            k, moe._cb)
+    print(f"moe two-launch tokens={tokens}", flush=True)
+    y1 = ops.moe_forward(*args, fused=True)
+    y2 = ops.moe_forward(*args, fused=True)
+    y5 = ops.moe_forward(*args, fused=False)
+    assert torch.equal(y1, y2)
+    ref = _oracle_chain(oracle, gate, up, down, x, idx, "silu")
+    assert rel_l2(y1.cpu().numpy(), ref) <= TOL
+    assert rel_l2(y5.cpu().numpy(), ref) <= TOL
+    assert rel_l2(y1.cpu().numpy(), y5.cpu().numpy()) <= TOL
+
+
 def test_moe_equals_linear_modules(cuda):
     """The stacked chain equals the same experts run as individual EXL3Linear
     modules (fused-vs-unfused, ponyexl3/tests/test_moe_activation.py:44-65)."""
