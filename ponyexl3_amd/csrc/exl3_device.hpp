@@ -93,18 +93,32 @@ __device__ __forceinline__ uint32_t scramble(uint32_t cw) {
     return __builtin_amdgcn_bitop3_b32(x, 0x8FFF8FFFu, 0x3B603B60u, 0x6A);  // c ^ (a & b)
 }
 
-// (half(x0.lo) + half(x0.hi), half(x1.lo) + half(x1.hi)) as a packed half2.
-__device__ __forceinline__ half2_t add_halves_pack(uint32_t x0, uint32_t x1) {
-    uint32_t r;
-    asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 "
-        "src1_sel:WORD_1"
-        : "=v"(r)
-        : "v"(x0));
-    asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 "
-        "src1_sel:WORD_1"
-        : "+v"(r)
-        : "v"(x1));
-    return bits_to_half2(r);
+// Two packed pairs at once:
+//   ra = (half(x0.lo) + half(x0.hi), half(x1.lo) + half(x1.hi)), rb likewise from x2, x3.
+// A VALU instruction that writes only half of a VGPR (SDWA dst_sel, here also the
+// UNUSED_PRESERVE read-modify-write of the second add) must be separated by one
+// wait state from any VALU or MFMA instruction that reads that VGPR on gfx950;
+// the compiler inserts those for its own instructions but cannot see inside
+// inline assembly. The block therefore interleaves the two pairs (each register
+// is touched every other instruction) and ends with one s_nop, so whatever the
+// scheduler places behind it is far enough away. Measured without it: an MFMA
+// issued right after the add read a stale upper half.
+__device__ __forceinline__ void add_halves_pack2(uint32_t x0, uint32_t x1, uint32_t x2,
+                                                 uint32_t x3, half2_t& ra, half2_t& rb) {
+    uint32_t a, b;
+    asm("v_add_f16_sdwa %0, %2, %2 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 "
+        "src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %1, %4, %4 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 "
+        "src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %0, %3, %3 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 "
+        "src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %1, %5, %5 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 "
+        "src1_sel:WORD_1\n\t"
+        "s_nop 0"
+        : "=&v"(a), "=&v"(b)
+        : "v"(x0), "v"(x1), "v"(x2), "v"(x3));
+    ra = bits_to_half2(a);
+    rb = bits_to_half2(b);
 }
 
 __device__ __forceinline__ half_t decode_mul1(uint32_t cw) {
@@ -114,16 +128,18 @@ __device__ __forceinline__ half_t decode_mul1(uint32_t cw) {
     return (half_t)v;
 }
 
-// Two codewords -> two packed fp16 weights.
+// Four codewords -> two packed pairs of fp16 weights (cw0, cw1) and (cw2, cw3).
 template <int CB>
-__device__ __forceinline__ half2_t decode_pair(uint32_t cw0, uint32_t cw1) {
+__device__ __forceinline__ void decode_pair2(uint32_t cw0, uint32_t cw1, uint32_t cw2,
+                                             uint32_t cw3, half2_t& ra, half2_t& rb) {
     if constexpr (CB == CB_MUL1) {
-        half2_t v;
-        v.x = decode_mul1(cw0);
-        v.y = decode_mul1(cw1);
-        return v;
+        ra.x = decode_mul1(cw0);
+        ra.y = decode_mul1(cw1);
+        rb.x = decode_mul1(cw2);
+        rb.y = decode_mul1(cw3);
     } else {
-        return add_halves_pack(scramble<CB>(cw0), scramble<CB>(cw1));
+        add_halves_pack2(scramble<CB>(cw0), scramble<CB>(cw1), scramble<CB>(cw2),
+                         scramble<CB>(cw3), ra, rb);
     }
 }
 
@@ -194,11 +210,12 @@ __device__ __forceinline__ LaneWords<K> finish_lane_words(const uint32_t (&own)[
 // multiplies x[2j], x[2j+1] with j = q + 4*hi.
 template <int K, int CB>
 __device__ __forceinline__ void decode_lane(const LaneWords<K>& lw, half2_t (&wp)[16]) {
-    static_for<0, 16>([&](auto pi) {
-        constexpr int n = 2 * pi.value;  // even codeword of the pair
-        constexpr int cs = cw_col_sel(n);
-        constexpr int j = cw_row(n) >> 1;  // x pair index
-        wp[8 * cs + j] = decode_pair<CB>(lane_codeword<K, n>(lw), lane_codeword<K, n + 1>(lw));
+    static_for<0, 8>([&](auto pj) {
+        constexpr int na = 4 * pj.value, nb = na + 2;  // even codewords of two consecutive pairs
+        constexpr int ia = 8 * cw_col_sel(na) + (cw_row(na) >> 1);
+        constexpr int ib = 8 * cw_col_sel(nb) + (cw_row(nb) >> 1);
+        decode_pair2<CB>(lane_codeword<K, na>(lw), lane_codeword<K, na + 1>(lw),
+                         lane_codeword<K, nb>(lw), lane_codeword<K, nb + 1>(lw), wp[ia], wp[ib]);
     });
 }
 

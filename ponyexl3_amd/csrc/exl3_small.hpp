@@ -81,16 +81,32 @@ __device__ __forceinline__ void stream_block_rows(const uint32_t* __restrict__ b
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
     };
+    // The dot products run on the matrix pipe, which works in the shadow of the
+    // decode VALU stream: v_mfma_f32_4x4x4_16b_f16 multiplies, in each of its 16
+    // independent blocks of 4 lanes, a 4x4 A (lane i of the block supplies row i)
+    // with a 4x4 B (lane j supplies column j) and leaves D[0..3][j] in lane j.
+    // With A row i = activations of batch row 4q+i and B column j = four
+    // consecutive weights of lane j's own output column, every lane gets the dot
+    // products of its weights with four batch rows; no data crosses lanes.
+    constexpr int NQ = (MT + 3) / 4;  // groups of four batch rows
+    float4_t accv[2][NQ];
+#pragma unroll
+    for (int cs = 0; cs < 2; cs++)
+#pragma unroll
+        for (int q = 0; q < NQ; q++) accv[cs][q] = float4_t{0.f, 0.f, 0.f, 0.f};
     struct XTile {
-        uint4_t q[MT][2];
+        uint4_t q[NQ][2];
     };
+    const int xlane = lane & 3;
     auto load_x = [&](int row_in_block) {
         XTile t;
 #pragma unroll
-        for (int m = 0; m < MT; m++) {
+        for (int q = 0; q < NQ; q++) {
+            int m = 4 * q + xlane;
+            if (m > MT - 1) m = MT - 1;  // rows past the batch repeat a staged row; never used
             const uint4_t* xp = reinterpret_cast<const uint4_t*>(&xw[m][row_in_block * 16]);
-            t.q[m][0] = xp[0];
-            t.q[m][1] = xp[1];
+            t.q[q][0] = xp[0];
+            t.q[q][1] = xp[1];
         }
         return t;
     };
@@ -99,15 +115,20 @@ __device__ __forceinline__ void stream_block_rows(const uint32_t* __restrict__ b
         half2_t wp[16];
         decode_lane<K, CB>(lw, wp);
 #pragma unroll
-        for (int m = 0; m < MT; m++) {
-            const uint4_t x0 = xt.q[m][0], x1 = xt.q[m][1];
-            const half2_t xv[8] = {bits_to_half2(x0.x), bits_to_half2(x0.y), bits_to_half2(x0.z),
-                                   bits_to_half2(x0.w), bits_to_half2(x1.x), bits_to_half2(x1.y),
-                                   bits_to_half2(x1.z), bits_to_half2(x1.w)};
+        for (int q = 0; q < NQ; q++) {
+            const uint4_t x0 = xt.q[q][0], x1 = xt.q[q][1];
+            const uint2_t xa[4] = {uint2_t{x0.x, x0.y}, uint2_t{x0.z, x0.w}, uint2_t{x1.x, x1.y},
+                                   uint2_t{x1.z, x1.w}};
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                acc[m][0] = dot2(wp[j], xv[j], acc[m][0]);
-                acc[m][1] = dot2(wp[8 + j], xv[j], acc[m][1]);
+            for (int j4 = 0; j4 < 4; j4++) {  // input rows 4*j4 .. 4*j4+3 of the tile
+#pragma unroll
+                for (int cs = 0; cs < 2; cs++) {
+                    const uint2_t wb = {half2_to_bits(wp[8 * cs + 2 * j4]),
+                                        half2_to_bits(wp[8 * cs + 2 * j4 + 1])};
+                    accv[cs][q] = __builtin_amdgcn_mfma_f32_4x4x4f16(
+                        __builtin_bit_cast(half4_t, xa[j4]), __builtin_bit_cast(half4_t, wb),
+                        accv[cs][q], 0, 0, 0);
+                }
             }
         }
     };
@@ -136,6 +157,11 @@ __device__ __forceinline__ void stream_block_rows(const uint32_t* __restrict__ b
             __builtin_amdgcn_sched_barrier(0);
             prev = prev_next;
         }
+    }
+#pragma unroll
+    for (int m = 0; m < MT; m++) {
+        acc[m][0] += accv[0][m >> 2][m & 3];
+        acc[m][1] += accv[1][m >> 2][m & 3];
     }
 }
 

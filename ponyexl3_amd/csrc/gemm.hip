@@ -137,19 +137,22 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
     // Pair pi (0..15) of a lane = codewords 2pi, 2pi+1 = input rows (2j, 2j+1) of
     // column u + 8*cs with cs = (pi>>1)&1, j = (pi>>2) + 4*(pi&1). The four pairs
     // {2cs + hh + 4t, t = 0..3} are the 8 consecutive rows 8hh..8hh+7 of column cs:
-    // one 16-byte store. Element e = 4*quad + t of the decode order.
-    auto decode_element = [&](const LaneWords<K>& lw, auto e_c, uint4_t& quad, half_t* bdst) {
-        constexpr int e = decltype(e_c)::value;
+    // one 16-byte store. Element e = 4*quad + t of the decode order; two elements
+    // are decoded per call (see add_halves_pack2 for why).
+    auto decode_element2 = [&](const LaneWords<K>& lw, auto e_c, uint4_t& quad, half_t* bdst) {
+        constexpr int e = decltype(e_c)::value;  // even: elements e and e + 1
         constexpr int q = e >> 2, t = e & 3;
         constexpr int cs = q >> 1, hh = q & 1;
-        constexpr int pi = 2 * cs + hh + 4 * t;
-        const uint32_t d = half2_to_bits(
-            decode_pair<CB>(lane_codeword<K, 2 * pi>(lw), lane_codeword<K, 2 * pi + 1>(lw)));
-        if constexpr (t == 0) quad.x = d;
-        if constexpr (t == 1) quad.y = d;
-        if constexpr (t == 2) quad.z = d;
-        if constexpr (t == 3) {
-            quad.w = d;
+        constexpr int pa = 2 * cs + hh + 4 * t, pb = pa + 4;
+        half2_t da, db;
+        decode_pair2<CB>(lane_codeword<K, 2 * pa>(lw), lane_codeword<K, 2 * pa + 1>(lw),
+                         lane_codeword<K, 2 * pb>(lw), lane_codeword<K, 2 * pb + 1>(lw), da, db);
+        if constexpr (t == 0) {
+            quad.x = half2_to_bits(da);
+            quad.y = half2_to_bits(db);
+        } else {
+            quad.z = half2_to_bits(da);
+            quad.w = half2_to_bits(db);
             *reinterpret_cast<uint4_t*>(bdst + b_w[cs] + 8 * hh) = quad;
         }
     };
@@ -177,7 +180,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
         load_w(clamp_k(k_begin + 1), S1{});
         const LaneWords<K> lw = finish_lane_words<K>(w_reg[0], lane);
         uint4_t quad;
-        static_for<0, 16>([&](auto e) { decode_element(lw, e, quad, b_s); });
+        static_for<0, 8>([&](auto e2) {
+            decode_element2(lw, std::integral_constant<int, 2 * decltype(e2)::value>{}, quad, b_s);
+        });
         load_w(clamp_k(k_begin + 2), S0{});
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -222,7 +227,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
         const LaneWords<K> lw = finish_lane_words<K>(w_reg[s], lane);
         __builtin_amdgcn_sched_barrier(0);  // keeps the trellis load behind the direct loads
         load_w(clamp_k(k + 3), slot);
-        static_for<0, EPG>([&](auto e) { decode_element(lw, e, quad, bdst); });
+        static_for<0, EPG / 2>([&](auto e2) {
+            decode_element2(lw, std::integral_constant<int, 2 * decltype(e2)::value>{}, quad, bdst);
+        });
         __builtin_amdgcn_sched_barrier(0);
         static_for<0, G>([&](auto gi_c) {
             constexpr int gi = decltype(gi_c)::value;
@@ -239,8 +246,10 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
                 for (int j = 0; j < 4; j++) bf[j] = ldb(1, j);
             }
             if constexpr (gi + 1 < G)
-                static_for<(gi + 1) * EPG, (gi + 2) * EPG>(
-                    [&](auto e) { decode_element(lw, e, quad, bdst); });
+                static_for<(gi + 1) * EPG / 2, (gi + 2) * EPG / 2>([&](auto e2) {
+                    decode_element2(lw, std::integral_constant<int, 2 * decltype(e2)::value>{},
+                                    quad, bdst);
+                });
             __builtin_amdgcn_sched_barrier(0);
         });
         // Memory operations retire in order and at least one trellis load was issued

@@ -171,8 +171,12 @@ def test_single_slot_cache_computes_once(cuda):
 @pytest.mark.parametrize("k,n_in,n_out", [(4, 512, 384), (3, 1024, 256), (6, 2176, 640), (4, 5120, 1024)])
 def test_one_launch_layer_equals_three_launch_chain(cuda, rows, k, n_in, n_out):
     """The fused kernel (rotation + GEMV + last-wave reduction + output transform)
-    must reproduce the chained kernels bit for bit, call after call (its group
-    counters have to come back to zero every time)."""
+    against the chained kernels. Both add the same fp32 products, but cut the
+    reduction dimension at different tile rows, so the sums can differ in the last
+    fp32 bit and, rarely, flip an fp16 rounding before the output Hadamard: they
+    must agree to a few fp16 ulps of the largest output. The fused kernel must be
+    bit-identical call after call (fixed sum order; its group counters have to
+    come back to zero every time)."""
     from ponyexl3_amd import make_exl3_layer, ops
 
     layer = make_exl3_layer(k=k, in_features=n_in, out_features=n_out, seed=k + n_in, bias=True)
@@ -184,6 +188,9 @@ def test_one_launch_layer_equals_three_launch_chain(cuda, rows, k, n_in, n_out):
     for rep in range(3):
         x = torch.from_numpy(rng.standard_normal((rows, n_in)).astype(np.float16)).to(cuda)
         a = ops.linear_forward(x, tr, k, 0, suh, svh, bias, fused=True)
+        a2 = ops.linear_forward(x, tr, k, 0, suh, svh, bias, fused=True)
         b = ops.linear_forward(x, tr, k, 0, suh, svh, bias, fused=False)
-        assert torch.equal(a, b), f"rep {rep}"
+        assert torch.equal(a, a2), f"rep {rep}"
+        diff = float((a.float() - b.float()).abs().max())
+        assert diff <= 2e-3 * float(b.float().abs().max()), f"rep {rep}: {diff}"
     assert int(ops.sync_counters(cuda, 1).abs().sum()) == 0
