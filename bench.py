@@ -140,6 +140,8 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-extras", action="store_true", help="skip prefill GEMM and MoE figures")
     ap.add_argument("--unfused-qkv", action="store_true", help="run q, k, v as three launches")
+    ap.add_argument("--sweep", action="store_true",
+                    help="also time config 5: the layer at K in {2,3,5,6,8}, 3INST and MCG, 1/4/8 rows")
     args = ap.parse_args()
     global LAYER
     if args.unfused_qkv:
@@ -226,32 +228,22 @@ def main():
     value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
 
     # ---- roofline of the dominant kernel: the one-launch layer kernel (input
-    # Hadamard + decode GEMV + split reduction + output Hadamard), timed per
-    # launch with HIP events on the launch stream
+    # Hadamard + decode GEMV + split reduction + output Hadamard). Its launch
+    # duration is measured per linear with two HIP events around back-to-back
+    # graph replays; a graph holds one launch per weight copy, with enough seeded
+    # copies of that linear (>= 320 MB) that no launch finds its weights in the
+    # 256 MB last-level cache. Durations measured this way agree with rocprofv3's
+    # per-dispatch figures to about a microsecond (the gap between dependent
+    # launches), see profiles/.
     per_linear = {}
-    reps = max(50, min(200, args.steps))
     tot_bytes = tot_ms = 0.0
-    # 1 GiB streamed between timed launches pushes the previous weights out of
-    # the 256 MB last-level cache (the same linear of 4 layer copies would fit)
-    flush = torch.zeros(1 << 30, dtype=torch.int8, device=dev)
     for j, (name, n_in, outs) in enumerate(LAYER):
-        lins = [layers[L][j] for L in range(n_layers)]
-        for r in range(10):
-            lins[r % n_layers].forward(xs[n_in])
-        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
-        torch.cuda.synchronize()
-        for r in range(reps):
-            flush.add_(1)
-            evs[r][0].record()
-            lins[r % n_layers].forward(xs[n_in])
-            evs[r][1].record()
-        torch.cuda.synchronize()
-        ms = float(np.mean([a.elapsed_time(b) for a, b in evs]))
-        per_linear[name] = {"MB": round(lins[0].bytes / 1e6, 2), "us": round(ms * 1e3, 2),
-                            "GBps": round(lins[0].bytes / ms / 1e6, 1)}
-        tot_bytes += lins[0].bytes
+        ms = _launch_ms(layers[0][j], xs[n_in], K_BITS, dev)
+        nb = layers[0][j].bytes
+        per_linear[name] = {"MB": round(nb / 1e6, 2), "us": round(ms * 1e3, 2),
+                            "GBps": round(nb / ms / 1e6, 1)}
+        tot_bytes += nb
         tot_ms += ms
-    del flush
     achieved = tot_bytes / tot_ms / 1e6
     roofline = {
         "bound": "hbm",
@@ -268,8 +260,12 @@ def main():
 
     extras = {}
     if not args.skip_extras:
+        extras.update(bench_batch_rows(dev, layers[0]))
+        extras.update(bench_config1(dev))
         extras.update(bench_prefill(dev, layers[0], xs))
         extras.update(bench_moe(dev))
+    if args.sweep:
+        extras.update(bench_sweep(dev, layers[0]))
 
     out = {
         "metric": "EXL3 GEMV effective GB/s (% HBM peak) at bs1; prefill GEMM TFLOPS at M=2048",
@@ -316,6 +312,31 @@ def _time_ms(fn, reps, warm=3):
     return float(np.mean([a.elapsed_time(b) for a, b in evs]))
 
 
+def _launch_ms(lin, x, k, dev, cb=CB, min_bytes=320e6, reps=20):
+    """Mean duration of one layer-kernel launch of the linear `lin` (its shape,
+    signs and sibling table) with K = k on cold weights: one graph of one launch
+    per seeded weight copy, replayed back to back between two HIP events."""
+    import torch
+
+    from ponyexl3_amd import ops
+
+    nbytes = lin.n_in * lin.n_out * k // 8
+    copies = max(2, int(np.ceil(min_bytes / nbytes)))
+    gen = torch.Generator(device=dev).manual_seed(31_000 + lin.n_in + lin.n_out + k)
+    trs = [torch.randint(-32768, 32768, (lin.n_in // 16, lin.n_out // 16, 16 * k), dtype=torch.int16,
+                         device=dev, generator=gen) for _ in range(copies)]
+    call = lambda tr: ops.linear_forward(x, tr, k, cb, lin.suh, lin.svh, None, lin.group_sub)
+    for tr in trs:
+        call(tr)
+    torch.cuda.synchronize()
+    gr = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(gr):
+        keep = [call(tr) for tr in trs]
+    ms = _time_batch_ms(gr.replay, reps=reps, warm=3) / copies
+    del gr, keep, trs
+    return ms
+
+
 def _time_batch_ms(fn, reps, warm=10):
     """Mean time of back-to-back calls (the queue never drains, so launch latency
     of an idle device is not part of it)."""
@@ -331,6 +352,47 @@ def _time_batch_ms(fn, reps, warm=10):
     b.record()
     torch.cuda.synchronize()
     return a.elapsed_time(b) / reps
+
+
+def _rows_x(n, rows, dev):
+    import torch
+
+    g = torch.Generator().manual_seed(4321 + n + rows)
+    return torch.randn((rows, n), generator=g).to(torch.float16).to(dev)
+
+
+def bench_batch_rows(dev, layer):
+    """The same layer step at 2, 4 and 8 rows (batched decode, speculative verify):
+    sum of the four launch durations on cold weights."""
+    res = {}
+    total = sum(l.bytes for l in layer)
+    for rows in (2, 4, 8):
+        ms = sum(_launch_ms(lin, _rows_x(lin.n_in, rows, dev), K_BITS, dev) for lin in layer)
+        res[f"rows_{rows}"] = {"us_per_step": round(ms * 1e3, 2), "GBps": round(total / ms / 1e6, 1)}
+    return {"batch_rows": res}
+
+
+def bench_config1(dev):
+    """config 1: one 4096 -> 4096 linear, K=4, 3INST, one row."""
+    lin = DeviceLinear("cfg1", 4096, [4096], 10_004, dev)
+    ms = _launch_ms(lin, _rows_x(4096, 1, dev), K_BITS, dev)
+    return {"config1": {"MB": round(lin.bytes / 1e6, 2), "us": round(ms * 1e3, 2),
+                        "GBps": round(lin.bytes / ms / 1e6, 1)}}
+
+
+def bench_sweep(dev, layer):
+    """config 5: the config-2 layer at other bit widths and codebooks, 1/4/8 rows."""
+    res = {}
+    for k in (2, 3, 5, 6, 8):
+        total = sum(l.n_in * l.n_out * k // 8 for l in layer)
+        for cb, cbn in ((0, "3inst"), (1, "mcg")):
+            for rows in (1, 4, 8):
+                ms = sum(_launch_ms(lin, _rows_x(lin.n_in, rows, dev), k, dev, cb=cb) for lin in layer)
+                res[f"k{k}_{cbn}_rows{rows}"] = {"us_per_step": round(ms * 1e3, 2),
+                                                 "GBps": round(total / ms / 1e6, 1)}
+                print(f"sweep k={k} {cbn} rows={rows}: {ms * 1e3:.1f} us/step, {total / ms / 1e6:.0f} GB/s",
+                      file=sys.stderr, flush=True)
+    return {"config5": res}
 
 
 def bench_prefill(dev, layer, xs):
@@ -351,7 +413,14 @@ def bench_prefill(dev, layer, xs):
         ms_tot += ms
         del xh
     tf = flop / ms_tot / 1e9
+    # context: what a plain fp16 GEMM of the library reaches on this box at the gate+up shape
+    a = torch.randn((2048, 5120), generator=g).to(torch.float16).to(dev)
+    b = torch.randn((5120, 34816), generator=g).to(torch.float16).to(dev)
+    ms_lib = _time_ms(lambda: torch.matmul(a, b), reps=10)
+    lib_tf = 2.0 * 2048 * 5120 * 34816 / ms_lib / 1e9
+    del a, b
     return {"prefill_gemm": {"M": 2048, "TFLOPs": round(tf, 1), "peak": MFMA_F16_PEAK_TFLOPS,
+                             "library_fp16_gemm_TFLOPs_gate_up_shape": round(lib_tf, 1),
                              "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "bound": "mfma",
                              "kernel": "gemm_kernel<K=4, cb=3INST>", "per_linear": per}}
 

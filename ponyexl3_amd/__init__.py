@@ -23,6 +23,8 @@ __all__ = [
     "FusedEXL3Sibling",
     "EXL3SwitchGLU",
     "fusable",
+    "reconstruct_inner",
+    "reconstruct_public_weights",
 ]
 
 
@@ -40,4 +42,8 @@ def __getattr__(name):
         from . import moe
 
         return getattr(moe, name)
+    if name in ("reconstruct_inner", "reconstruct_public_weights"):
+        from . import ops
+
+        return getattr(ops, name)
     raise AttributeError(name)

@@ -137,6 +137,46 @@ def decode_full(trellis, k: int, cb: int, tn_offset: int = 0, tn_count: int | No
     return w
 
 
+def reconstruct_inner(trellis, k: int, cb: int, n_offset: int = 0, n_count: int | None = None):
+    """Inner weight W (in, n_count) fp16 for a 128-aligned column range
+    (``reconstruct_inner``, ponyexl3/ref/reconstruct.py:13-23; the reference
+    rejects unaligned offsets the same way, ref/decode.py:46-51)."""
+    _, out_tiles = _trellis_dims(trellis, k)
+    if n_count is None:
+        n_count = out_tiles * 16 - n_offset
+    if n_offset % 128 or n_count % 16 or n_offset < 0 or n_count < 0:
+        raise ValueError("column slice must start on a multiple of 128 and cover whole tiles")
+    return decode_full(trellis, k, cb, n_offset // 16, n_count // 16)
+
+
+def _hadamard128_matrix(device) -> torch.Tensor:
+    h = torch.ones((1, 1), dtype=torch.float32, device=device)
+    while h.shape[0] < 128:
+        h = torch.cat([torch.cat([h, h], dim=1), torch.cat([h, -h], dim=1)], dim=0)
+    return h * (128.0 ** -0.5)
+
+
+def reconstruct_public_weights(trellis, suh, svh, k: int, cb: int):
+    """Public weight diag(suh) . H . W . H . diag(svh), fp32 arithmetic, one cast to
+    fp16 (``reconstruct_public_weights``, ponyexl3/ref/reconstruct.py:26-49). The
+    decode runs in the HIP kernel; the two blockwise Hadamard products are plain
+    torch matmuls, this is a checking and export utility, not a forward path."""
+    w = decode_full(trellis, k, cb).float()
+    n_in, n_out = w.shape
+    h = _hadamard128_matrix(w.device)
+    if suh is not None:
+        if n_in % 128:
+            raise ValueError(f"in_features {n_in} not divisible by 128")
+        w = torch.matmul(h, w.reshape(n_in // 128, 128, n_out)).reshape(n_in, n_out)
+        w = w * suh.to(w.device).float().reshape(-1, 1)
+    if svh is not None:
+        if n_out % 128:
+            raise ValueError(f"out_features {n_out} not divisible by 128")
+        w = torch.matmul(w.reshape(n_in, n_out // 128, 128), h).reshape(n_in, n_out)
+        w = w * svh.to(w.device).float().reshape(1, -1)
+    return w.to(torch.float16)
+
+
 def had128_pre(x2d: torch.Tensor, suh: torch.Tensor | None):
     """xh = fp16(had128(x * suh)); suh (in,) or stacked (n_sub, in) -> xh
     (rows, in) or (rows, n_sub, in). ``EXL3LayerRuntime.prepare_xh`` /

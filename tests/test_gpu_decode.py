@@ -3,7 +3,7 @@ import numpy as np
 import pytest
 import torch
 
-from conftest import golden
+from conftest import golden, rel_l2
 
 pytestmark = pytest.mark.gpu
 
@@ -68,3 +68,29 @@ def test_errors(cuda):
         ops.decode_full(tr, 4, 0, tn_offset=2, tn_count=2)
     with pytest.raises(ValueError):
         ops.decode_full(tr, 4, 5)
+
+
+def test_reconstruct_public_weights(cuda, oracle):
+    """diag(suh).H.W.H.diag(svh) against the oracle (ref/reconstruct.py:26-49), and
+    the reference's own check that x @ W_pub reproduces the layer forward
+    (tests/test_decode_reconstruct.py:40-69)."""
+    from ponyexl3_amd import EXL3Linear, make_exl3_layer, ops
+
+    layer = make_exl3_layer(k=3, in_features=256, out_features=384, seed=77, mcg=True)
+    tr = ops.as_trellis_tensor(layer.trellis, cuda)
+    suh, svh = torch.from_numpy(layer.suh).to(cuda), torch.from_numpy(layer.svh).to(cuda)
+    w_pub = ops.reconstruct_public_weights(tr, suh, svh, 3, int(layer.codebook_mode))
+    ref = oracle.reconstruct_public_weights(layer.trellis, layer.suh, layer.svh, 3, int(layer.codebook_mode))
+    assert w_pub.dtype == torch.float16 and tuple(w_pub.shape) == (256, 384)
+    assert rel_l2(w_pub.cpu().numpy(), ref) < 1e-3
+    inner = ops.reconstruct_inner(tr, 3, int(layer.codebook_mode), n_offset=128, n_count=128)
+    np.testing.assert_array_equal(
+        inner.cpu().numpy().view(np.uint16),
+        oracle.decode_trellis(layer.trellis, 3, int(layer.codebook_mode), tn_offset=8, tn_count=8).view(np.uint16))
+    rng = np.random.default_rng(5)
+    x = torch.from_numpy(rng.standard_normal((4, 256)).astype(np.float16)).to(cuda)
+    y = EXL3Linear(layer)(x).float()
+    y_pub = x.float() @ w_pub.float()
+    assert float((y - y_pub).norm() / y_pub.norm()) < 5e-3
+    with pytest.raises(ValueError):
+        ops.reconstruct_inner(tr, 3, int(layer.codebook_mode), n_offset=64)
