@@ -1,10 +1,16 @@
 // Hadamard-128 regularisation kernels (input side with suh, output side with
 // split-K reduction + svh + bias).
 //
-// One wavefront owns one 128-wide block: lane l holds elements 2l and 2l+1 in
-// fp32. The Sylvester transform factors into 7 butterfly stages that commute;
-// the stage on element bit 0 is in-lane, the other six exchange with lane
-// l ^ (1 << b). No LDS, no barriers. Arithmetic follows
+// Narrow form (few rows, fp32 partial sums): one wavefront owns one 128-wide
+// block, lane l holds elements 2l and 2l+1 in fp32. The Sylvester transform
+// factors into 7 butterfly stages that commute; the stage on element bit 0 is
+// in-lane, the other six exchange with lane l ^ (1 << b).
+// Wide form (prefill, fp16 in and out): lane l of a 16-lane group holds the 8
+// consecutive elements 8l..8l+7 of a block (one 16-byte load), the stages on
+// element bits 0..2 are in-lane and the other four exchange inside the group, so
+// a wavefront transforms four blocks per 1 KiB load and a workgroup walks along
+// one row. Same stage order and the same a+b / a-b per stage as the narrow form,
+// hence the same bits. No LDS, no barriers. Arithmetic follows
 // ponyexl3/ref/hadamard.py:50-80: multiply by the pre vector in fp32,
 // transform, scale by 1/sqrt(128), multiply by the post vector in fp32, and the
 // caller-visible casts of ponyexl3/ref/forward.py:34,41,42,45.
@@ -29,6 +35,113 @@ __device__ __forceinline__ void wht128(float& a, float& b, int lane) {
         const bool upper = (lane & mask) != 0;
         a = upper ? pa - a : a + pa;
         b = upper ? pb - b : b + pb;
+    }
+}
+
+// v[j] = element 8*(lane & 15) + j of the lane group's block, unnormalised WHT in place.
+__device__ __forceinline__ void wht128_wide(float (&v)[8], int lane) {
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            if ((j & h) == 0) {
+                const float lo = v[j], hi = v[j + h];
+                v[j] = lo + hi;
+                v[j + h] = lo - hi;
+            }
+        }
+    }
+#pragma unroll
+    for (int bit = 0; bit < 4; bit++) {
+        const int mask = 1 << bit;
+        const bool upper = (lane & mask) != 0;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float p = __shfl_xor(v[j], mask, kWave);
+            v[j] = upper ? p - v[j] : v[j] + p;
+        }
+    }
+}
+
+__device__ __forceinline__ void halfs_to_floats(uint4_t q, float (&v)[8]) {
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const half2_t h = bits_to_half2(w[i]);
+        v[2 * i] = (float)h.x;
+        v[2 * i + 1] = (float)h.y;
+    }
+}
+
+// Wide forms: grid.x = number of output rows ((row, sub) pairs for the input side);
+// the four waves of a workgroup take consecutive 512-element chunks of the row.
+// All pointers 16-byte aligned, n a multiple of 128.
+__global__ __launch_bounds__(256) void had_pre_wide_kernel(const half_t* __restrict__ x,
+                                                           const half_t* __restrict__ suh,
+                                                           half_t* __restrict__ xh, int n,
+                                                           int n_sub) {
+    const int lane = threadIdx.x & 63;
+    const size_t rs = blockIdx.x;
+    const half_t* xr = x + (rs / n_sub) * (size_t)n;
+    const half_t* sr = suh ? suh + (rs % n_sub) * (size_t)n : nullptr;
+    half_t* orow = xh + rs * (size_t)n;
+    for (int c = threadIdx.x * 8; c < n; c += 2048) {
+        float v[8], sv[8];
+        halfs_to_floats(*reinterpret_cast<const uint4_t*>(xr + c), v);
+        if (sr) {
+            halfs_to_floats(*reinterpret_cast<const uint4_t*>(sr + c), sv);
+#pragma unroll
+            for (int j = 0; j < 8; j++) v[j] = v[j] * sv[j];
+        }
+        wht128_wide(v, lane);
+        uint4_t o;
+        uint32_t* ow = reinterpret_cast<uint32_t*>(&o);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            half2_t h;
+            h.x = (half_t)(v[2 * i] * kHadScale);
+            h.y = (half_t)(v[2 * i + 1] * kHadScale);
+            ow[i] = half2_to_bits(h);
+        }
+        *reinterpret_cast<uint4_t*>(orow + c) = o;
+    }
+}
+
+__global__ __launch_bounds__(256) void had_post_wide_kernel(const half_t* __restrict__ y,
+                                                            const half_t* __restrict__ svh,
+                                                            const half_t* __restrict__ bias,
+                                                            half_t* out, int n) {
+    const int lane = threadIdx.x & 63;
+    const half_t* yr = y + (size_t)blockIdx.x * n;
+    half_t* orow = out + (size_t)blockIdx.x * n;
+    for (int c = threadIdx.x * 8; c < n; c += 2048) {
+        float v[8], sv[8];
+        halfs_to_floats(*reinterpret_cast<const uint4_t*>(yr + c), v);
+        wht128_wide(v, lane);
+        if (svh) halfs_to_floats(*reinterpret_cast<const uint4_t*>(svh + c), sv);
+        uint4_t bq = {0u, 0u, 0u, 0u};
+        if (bias) bq = *reinterpret_cast<const uint4_t*>(bias + c);
+        const uint32_t* bw = reinterpret_cast<const uint32_t*>(&bq);
+        uint4_t o;
+        uint32_t* ow = reinterpret_cast<uint32_t*>(&o);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float a = v[2 * i] * kHadScale, b = v[2 * i + 1] * kHadScale;
+            if (svh) {
+                a = a * sv[2 * i];
+                b = b * sv[2 * i + 1];
+            }
+            half2_t h;
+            h.x = (half_t)a;
+            h.y = (half_t)b;
+            if (bias) {
+                const half2_t bv = bits_to_half2(bw[i]);
+                h.x = h.x + bv.x;
+                h.y = h.y + bv.y;
+            }
+            ow[i] = half2_to_bits(h);
+        }
+        *reinterpret_cast<uint4_t*>(orow + c) = o;
     }
 }
 
@@ -123,6 +236,11 @@ __global__ __launch_bounds__(256) void had_post_kernel(const void* __restrict__ 
     *reinterpret_cast<half2_t*>(out + off) = o;
 }
 
+// From this many rows on the wide kernels (one workgroup per row) fill the device
+// better than one wave per 128-element block.
+constexpr int kWideMinRows = 16;
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
 int launch_had_pre(const uint16_t* x, int rows, int n, const uint16_t* suh, int n_sub,
                    uint16_t* xh, hipStream_t stream) {
     if (!x || !xh) return EXL3_E_NULL_POINTER;
@@ -132,6 +250,13 @@ int launch_had_pre(const uint16_t* x, int rows, int n, const uint16_t* suh, int 
     const long long waves = (long long)rows * n_sub * (n / 128);
     const long long grid = (waves + 3) / 4;
     if (grid > 0x7FFFFFFFLL) return EXL3_E_BAD_SHAPE;
+    if ((long long)rows * n_sub >= kWideMinRows && aligned16(x) && aligned16(xh) &&
+        (!suh || aligned16(suh))) {
+        had_pre_wide_kernel<<<dim3((unsigned)(rows * n_sub)), dim3(256), 0, stream>>>(
+            reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(suh),
+            reinterpret_cast<half_t*>(xh), n, n_sub);
+        return launch_status();
+    }
     had_pre_kernel<<<dim3((unsigned)grid), dim3(256), 0, stream>>>(
         reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(suh),
         reinterpret_cast<half_t*>(xh), rows, n, n_sub);
@@ -150,6 +275,12 @@ int launch_had_post(const void* y, int y_is_fp32, int n_sum, size_t sum_stride, 
     const half_t* s = reinterpret_cast<const half_t*>(svh);
     const half_t* b = reinterpret_cast<const half_t*>(bias);
     half_t* o = reinterpret_cast<half_t*>(out);
+    if (!y_is_fp32 && rows >= kWideMinRows && aligned16(y) && aligned16(out) &&
+        (!svh || aligned16(svh)) && (!bias || aligned16(bias))) {
+        had_post_wide_kernel<<<dim3((unsigned)rows), dim3(256), 0, stream>>>(
+            reinterpret_cast<const half_t*>(y), s, b, o, n);
+        return launch_status();
+    }
     if (y_is_fp32)
         had_post_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, stream>>>(y, n_sum, sum_stride,
                                                                               s, b, o, rows, n);

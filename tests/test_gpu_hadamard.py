@@ -59,6 +59,29 @@ def test_post_fp16_and_split_sum(cuda, oracle):
     np.testing.assert_array_equal(gotb.view(np.uint16), (got16 + bias).view(np.uint16))
 
 
+def test_wide_and_narrow_kernels_give_the_same_bits(cuda, oracle):
+    """From 16 rows on a workgroup walks along a row with 16-byte accesses; below,
+    one wave takes one block. Same butterflies in the same order: same bits."""
+    from ponyexl3_amd import ops
+
+    rng = np.random.default_rng(4)
+    x = (rng.standard_normal((40, 640)) * 3).astype(np.float16)
+    suh = (np.where(rng.random((3, 640)) > 0.5, -1, 1) * rng.uniform(0.5, 2, (3, 640))).astype(np.float16)
+    svh = (np.where(rng.random(640) > 0.5, -1, 1) * rng.uniform(0.5, 2, 640)).astype(np.float16)
+    bias = (rng.standard_normal(640) * 0.1).astype(np.float16)
+    xt, st, vt, bt = _t(x, cuda), _t(suh, cuda), _t(svh, cuda), _t(bias, cuda)
+    wide = ops.had128_pre(xt, st)  # 120 (row, sub) pairs: wide kernel
+    narrow = torch.cat([ops.had128_pre(xt[r:r + 5].contiguous(), st) for r in range(0, 40, 5)])
+    assert torch.equal(wide, narrow)
+    ref = oracle.had_r_128(x.astype(np.float32), pre_scale=suh[1]).astype(np.float16)
+    assert rel_l2(wide[:, 1].cpu().numpy(), ref) < 3e-4
+    wide = ops.had128_post(xt, vt, bt)
+    narrow = torch.cat([ops.had128_post(xt[r:r + 8].contiguous(), vt, bt) for r in range(0, 40, 8)])
+    assert torch.equal(wide, narrow)
+    ref = oracle.had_r_128(x.astype(np.float32), post_scale=svh).astype(np.float16)
+    assert rel_l2(ops.had128_post(xt, vt).cpu().numpy(), ref) < 3e-4
+
+
 def test_involution_at_scale(cuda):
     """Size-independent property at prefill size: H(H(x)) == x, norms preserved."""
     from ponyexl3_amd import ops
