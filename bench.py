@@ -87,11 +87,13 @@ class DeviceLinear:
             gs = np.repeat(np.arange(members, dtype=np.int32), [o // 128 for o in outs])
             self.group_sub = torch.from_numpy(gs).to(device)
         self.bytes = weight_bytes(n_in, outs)
+        self.outs = list(outs)
 
     def forward(self, x):
         from ponyexl3_amd import ops
 
-        return ops.linear_forward(x, self.trellis, K_BITS, CB, self.suh, self.svh, None, self.group_sub)
+        return ops.linear_forward(x, self.trellis, K_BITS, CB, self.suh, self.svh, None, self.group_sub,
+                                  member_out=self.outs if self.members > 1 else None)
 
 
 def cpu_baseline(budget_s=12.0):
@@ -403,14 +405,18 @@ def bench_prefill(dev, layer, xs):
 
     g = torch.Generator().manual_seed(77)
     per = {}
-    flop = ms_tot = 0.0
+    flop = ms_tot = ms_layer_tot = 0.0
     for lin in layer:
         xh = torch.randn((2048, lin.n_in), generator=g).to(torch.float16).to(dev)
         ms = _time_ms(lambda: ops.inner_gemm(xh, lin.trellis, K_BITS, CB), reps=10)
+        # the whole layer at 2048 rows: input Hadamard, GEMM, output Hadamard
+        ms_layer = _time_ms(lambda: lin.forward(xh), reps=10)
         f = 2.0 * 2048 * lin.n_in * lin.n_out
-        per[lin.name] = {"ms": round(ms, 4), "TFLOPs": round(f / ms / 1e9, 1)}
+        per[lin.name] = {"ms": round(ms, 4), "TFLOPs": round(f / ms / 1e9, 1),
+                         "layer_ms": round(ms_layer, 4), "layer_TFLOPs": round(f / ms_layer / 1e9, 1)}
         flop += f
         ms_tot += ms
+        ms_layer_tot += ms_layer
         del xh
     tf = flop / ms_tot / 1e9
     # context: what a plain fp16 GEMM of the library reaches on this box at the gate+up shape
@@ -420,6 +426,7 @@ def bench_prefill(dev, layer, xs):
     lib_tf = 2.0 * 2048 * 5120 * 34816 / ms_lib / 1e9
     del a, b
     return {"prefill_gemm": {"M": 2048, "TFLOPs": round(tf, 1), "peak": MFMA_F16_PEAK_TFLOPS,
+                             "layer_TFLOPs_with_hadamards": round(flop / ms_layer_tot / 1e9, 1),
                              "library_fp16_gemm_TFLOPs_gate_up_shape": round(lib_tf, 1),
                              "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "bound": "mfma",
                              "kernel": "gemm_kernel<K=4, cb=3INST>", "per_linear": per}}

@@ -67,28 +67,10 @@ class FusedEXL3Group(torch.nn.Module):
     def forward_all(self, x: torch.Tensor) -> tuple[torch.Tensor, ...]:
         lead = tuple(x.shape[:-1])
         x2d = x.reshape(-1, self.in_features).to(torch.float16).contiguous()
-        rows = x2d.shape[0]
-        total_out = sum(self._out_features)
-        if rows <= ops.gemv_max_rows():
-            y = ops.linear_forward(
-                x2d, self._trellis, self._k, self._cb, self._suh_stack, self._svh_cat, None,
-                self._group_sub,
-            )
-        else:
-            # prefill: one MFMA GEMM per member over its tile-column range, each
-            # reading its own rotated activations out of the stacked buffer
-            xh = ops.had128_pre(x2d, self._suh_stack)  # (rows, n_sub, in)
-            n_sub = len(self._out_features)
-            yraw = torch.empty((rows, total_out), dtype=torch.float16, device=x2d.device)
-            tn0 = 0
-            for i, n in enumerate(self._out_features):
-                ops.gemm_into(
-                    xh.data_ptr() + 2 * i * self.in_features, rows, n_sub * self.in_features,
-                    self._trellis, self._k, self._cb, tn0, n // 16,
-                    yraw.data_ptr() + 2 * 16 * tn0, total_out, x2d.device,
-                )
-                tn0 += n // 16
-            y = ops.had128_post(yraw, self._svh_cat)
+        y = ops.linear_forward(
+            x2d, self._trellis, self._k, self._cb, self._suh_stack, self._svh_cat, None,
+            self._group_sub, member_out=self._out_features,
+        )
         outs = torch.split(y, self._out_features, dim=-1)
         return tuple(o.reshape(lead + (n,)) for o, n in zip(outs, self._out_features))
 

@@ -377,9 +377,13 @@ def gemm_into(xh_ptr: int, rows: int, ldx: int, trellis, k: int, cb: int, tn_off
 
 
 def linear_forward(x2d, trellis, k, cb, suh=None, svh=None, bias=None, group_sub=None,
-                   fused: bool = True):
+                   fused: bool = True, member_out=None):
     """Whole-layer forward on (rows, in) fp16 (``exl3_linear_forward``).
-    ``fused=False`` selects the three-launch chain for small batches."""
+    ``fused=False`` selects the three-launch chain for small batches.
+    ``member_out`` (out_features of each sibling, in order) is needed for a
+    sibling-fused group above ``gemv_max_rows()`` rows: the prefill GEMM runs once
+    per member over its tile columns, each on its own rotated activations
+    (``FusedEXL3Group.forward_all``, ponyexl3/mlx/exl3_fused.py:136-202)."""
     in_tiles, out_tiles = _trellis_dims(trellis, k)
     _half(x2d, "x")
     if x2d.dim() != 2 or x2d.shape[1] != in_tiles * 16:
@@ -408,6 +412,18 @@ def linear_forward(x2d, trellis, k, cb, suh=None, svh=None, bias=None, group_sub
     y = torch.empty((rows, n_out), dtype=torch.float16, device=x2d.device)
     if rows == 0:
         return y
+    if n_sub > 1 and rows > gemv_max_rows():
+        if member_out is None or len(member_out) != n_sub or sum(member_out) != n_out:
+            raise ValueError("member_out must list the out_features of the stacked members")
+        xh = had128_pre(x2d, suh)  # (rows, n_sub, in)
+        tn0 = 0
+        for i, n in enumerate(member_out):
+            if n % 128:
+                raise ValueError("member out_features must be multiples of 128")
+            gemm_into(xh.data_ptr() + 2 * i * n_in, rows, n_sub * n_in, trellis, k, cb, tn0, n // 16,
+                      y.data_ptr() + 2 * 16 * tn0, n_out, x2d.device)
+            tn0 += n // 16
+        return had128_post(y, svh, bias)
     lib = _lib.load()
     ws_bytes = int(lib.exl3_linear_workspace_bytes(rows, n_in, n_out, n_sub))
     ws = workspace(x2d.device, ws_bytes)

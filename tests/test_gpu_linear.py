@@ -57,6 +57,31 @@ def test_module_matches_oracle(cuda, oracle, rows, k, mcg):
     assert rel_l2(y, _oracle_forward(oracle, layer, x)) <= TOL
 
 
+@pytest.mark.parametrize("k", [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("cb", [0, 1, 2])
+def test_every_k_codebook_and_row_count(cuda, oracle, k, cb):
+    """Every bit width, codebook and small-batch row count (each row count up to 8
+    is its own instruction schedule in the one-launch kernel), both launch plans,
+    plus two prefill row counts, against the oracle."""
+    from ponyexl3_amd import make_exl3_layer, ops
+
+    layer = make_exl3_layer(k=k, in_features=256, out_features=256, seed=300 + 10 * k + cb,
+                            mcg=cb == 1, mul1=cb == 2, bias=True)
+    tr = ops.as_trellis_tensor(layer.trellis, cuda)
+    suh, svh = torch.from_numpy(layer.suh).to(cuda), torch.from_numpy(layer.svh).to(cuda)
+    bias = torch.from_numpy(layer.bias).to(cuda)
+    rng = np.random.default_rng(k * 3 + cb)
+    for rows in (1, 2, 3, 4, 5, 6, 7, 8, 12, 70):
+        x, xt = _x(rng, (rows, 256), cuda)
+        ref = _oracle_forward(oracle, layer, x)
+        print(f"k={k} cb={cb} rows={rows}", flush=True)
+        y = ops.linear_forward(xt, tr, k, cb, suh, svh, bias, fused=True).cpu().numpy()
+        assert rel_l2(y, ref) <= TOL, f"one-launch rows={rows}"
+        if rows <= 8:
+            y = ops.linear_forward(xt, tr, k, cb, suh, svh, bias, fused=False).cpu().numpy()
+            assert rel_l2(y, ref) <= TOL, f"chain rows={rows}"
+
+
 def test_general_scales_not_only_signs(cuda, oracle):
     from ponyexl3_amd import EXL3Linear, make_exl3_layer
 
