@@ -12,10 +12,12 @@ several distinct copies of the layer so the weights come from HBM, not from the
 256 MB last-level cache. ``value`` is effective weight bytes per second over the
 whole step (Hadamard kernels and launch gaps included).
 
-Prints ONE JSON line (see README / DESIGN.md for the fields). Extra objects:
-roofline (dominant kernel = the decode GEMV, timed per launch with HIP events),
-cpu_baseline (the C oracle on the host cores), prefill_gemm (M=2048, config 3)
-and moe (config 4).
+Prints ONE JSON line: metric, value, unit, n_gpus, steps, warmup, ms_per_step,
+higher_is_better, scaling, vs_baseline, dtype, data, config, plus the objects
+roofline (dominant kernel = the one-launch layer kernel, launch durations from
+HIP events around batched graph replays on cold weights), cpu_baseline (the C
+oracle on the host cores), batch_rows (2/4/8 rows), config1, prefill_gemm
+(M=2048, config 3), moe (config 4) and, with --sweep, config5.
 """
 
 from __future__ import annotations

@@ -87,7 +87,7 @@ int launch_had_post(const void* y, int y_is_fp32, int n_sum, size_t sum_stride, 
 // round are cut into `split` reduction ranges of `ksteps_per_split` 64-deep steps
 // whose fp32 partial tiles a second kernel adds up.
 struct GemmPlan {
-    int mi;  // 16-row accumulator tiles per wave: 8 (256-row blocks) or 2 (64-row blocks)
+    int mi;  // 16-row accumulator tiles per wave: 8, 4 or 2 (256-, 128- or 64-row blocks)
     int n_row_blocks, n_col_blocks;
     int full_tiles, split_tiles;
     int split, ksteps_per_split;

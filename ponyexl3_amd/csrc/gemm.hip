@@ -2,8 +2,9 @@
 // contracted on fp16 MFMA (v_mfma_f32_16x16x32_f16), fp32 accumulation.
 //
 // One workgroup = 8 wavefronts (2 per SIMD), one workgroup per CU.
-//   block tile   BM x 256 columns, BK = 64 (four tile rows); BM = 256 (MI = 8) or
-//                64 (MI = 2, small batches: less padding work per decoded tile)
+//   block tile   BM x 256 columns, BK = 64 (four tile rows); BM = 256 (MI = 8),
+//                128 (MI = 4) or 64 (MI = 2) for small batches: less padding
+//                work per decoded tile
 //   wave tile    (BM/2) x 64 -> MI x 4 accumulator tiles of 16x16
 //   LDS          two stages of A [BM][64] and B [256][64] fp16 (128 KiB at MI = 8):
 //                stage s^1 is filled while stage s is contracted, one barrier per
@@ -349,7 +350,7 @@ static int gemm_slots() {
 
 GemmPlan plan_gemm(int rows, int in_tiles, int tn_count, bool allow_split) {
     GemmPlan p{};
-    p.mi = rows <= 64 ? 2 : 8;
+    p.mi = rows <= 64 ? 2 : rows <= 128 ? 4 : 8;
     const int bm = 32 * p.mi;
     p.n_row_blocks = (rows + bm - 1) / bm;
     p.n_col_blocks = (tn_count + 15) / 16;
@@ -435,6 +436,10 @@ int launch_gemm(const uint16_t* xh, int rows, size_t ldx, const uint16_t* trelli
     return dispatch_k_cb(K, cb, [&](auto k, auto c) {
         if (p.mi == 2)
             return launch_gemm_mi<k.value, c.value, 2>(p, xh, rows, ldx, trellis, in_tiles,
+                                                       out_tiles, tn_offset, tn_count, y_out, ldy,
+                                                       partial, stream);
+        if (p.mi == 4)
+            return launch_gemm_mi<k.value, c.value, 4>(p, xh, rows, ldx, trellis, in_tiles,
                                                        out_tiles, tn_offset, tn_count, y_out, ldy,
                                                        partial, stream);
         return launch_gemm_mi<k.value, c.value, 8>(p, xh, rows, ldx, trellis, in_tiles, out_tiles,

@@ -14,7 +14,7 @@ def _t(a, device):
     return torch.from_numpy(np.ascontiguousarray(a)).to(device)
 
 
-@pytest.mark.parametrize("rows", [9, 17, 256, 300, 513])
+@pytest.mark.parametrize("rows", [9, 17, 100, 256, 300, 513])
 @pytest.mark.parametrize("k,cb", [(4, 0), (3, 1), (5, 0), (8, 1), (1, 0), (7, 1), (4, 2)])
 def test_gemm_matches_oracle(cuda, oracle, rows, k, cb):
     from ponyexl3_amd import ops
@@ -73,7 +73,7 @@ def test_config3_prefill_against_decoded_weights(cuda, oracle):
     assert float(err) < 5e-4
 
 
-@pytest.mark.parametrize("rows", [40, 300])
+@pytest.mark.parametrize("rows", [40, 100, 300])
 def test_split_tiles_match_oracle_and_unsplit(cuda, oracle, rows):
     """Few tiles and a deep reduction: every tile is cut into reduction ranges
     whose fp32 partial tiles a second kernel adds. Checked against the oracle,
