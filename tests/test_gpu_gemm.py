@@ -41,6 +41,23 @@ def test_gemm_column_slice(cuda, oracle):
     assert rel_l2(y, xh.astype(np.float64) @ w) < 5e-4
 
 
+def test_slice_with_half_width_last_block_and_split_tiles(cuda, oracle):
+    """A column slice that starts inside the matrix, ends with a half-width
+    (128-column) block and is few enough tiles that every tile is split along the
+    reduction dimension; the columns outside the slice must stay untouched."""
+    from ponyexl3_amd import _lib, ops
+
+    rng = np.random.default_rng(45)
+    tr_np = rng.integers(0, 65536, size=(128, 48, 64), dtype=np.uint16)  # 2048 -> 768
+    tr = ops.as_trellis_tensor(tr_np, cuda)
+    xh_np = rng.standard_normal((300, 2048)).astype(np.float16)
+    assert _lib.load().exl3_gemm_workspace_bytes(300, 128, 24) > 0
+    y = ops.inner_gemm(_t(xh_np, cuda), tr, 4, 0, tn_offset=8, tn_count=24).cpu().numpy()
+    assert y.shape == (300, 384)
+    w = oracle.decode_trellis(tr_np, 4, 0, tn_offset=8, tn_count=24).astype(np.float64)
+    assert rel_l2(y, xh_np.astype(np.float64) @ w) < 5e-4
+
+
 def test_small_batch_and_prefill_kernels_agree(cuda):
     from ponyexl3_amd import ops
 
