@@ -499,6 +499,23 @@ def bench_moe(dev):
                               "distinct_experts": round(mean_distinct, 1),
                               "MB": round(nbytes / 1e6, 2), "GBps": round(nbytes / ms / 1e6, 1),
                               "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    # prefill: 512 tokens through the sorted, segmented GEMM path (eager launches,
+    # host-side sort and table ops included)
+    T = 512
+    x = torch.from_numpy((rng.standard_normal((1, T, D)) * 0.25).astype(np.float16)).to(dev)
+    logits = torch.from_numpy(rng.standard_normal((T, E)).astype(np.float32)).to(dev)
+    inds, _ = route_topk(logits, kk)
+    idx = inds.reshape(1, T, kk).to(torch.int32).contiguous()
+    it = [0]
+
+    def prefill():
+        moes[it[0] % copies](x, idx)
+        it[0] += 1
+
+    ms = _time_batch_ms(prefill, reps=10, warm=3)
+    flop = 2.0 * T * kk * 3 * D * H
+    res["tokens_512_prefill"] = {"ms": round(ms, 4), "TFLOPs": round(flop / ms / 1e9, 1),
+                                 "expert_weights_MB": round(E * 3 * D * H * K_BITS / 8 / 1e6, 1)}
     return {"moe": res}
 
 

@@ -86,6 +86,15 @@ int exl3_had128_pre(const uint16_t *x, int rows, int n, const uint16_t *suh, int
  *   svh, bias   fp16 [n] or NULL
  *   out         fp16 [rows][n]; may alias y when y is fp16
  */
+/*
+ * Hadamard-128 with one scale vector per row (rows routed to different experts):
+ *   post == 0: out = fp16(had128(x * scale_rows))   (_rows_prep, ponyexl3/mlx/exl3_moe.py:105-119)
+ *   post != 0: out = fp16(had128(x) * scale_rows)   (_rows_finish, ponyexl3/mlx/exl3_moe.py:122-136)
+ * x, scale_rows, out fp16 [rows][n], 16-byte aligned, n a multiple of 128.
+ */
+int exl3_had128_rows(const uint16_t *x, int rows, int n, const uint16_t *scale_rows, int post,
+                     uint16_t *out, void *stream);
+
 int exl3_had128_post(const void *y, int y_is_fp32, int n_sum, size_t sum_stride, int rows, int n,
                      const uint16_t *svh, const uint16_t *bias, uint16_t *out, void *stream);
 
@@ -151,6 +160,25 @@ int exl3_gemv_partials(const uint16_t *xh, int rows, int n_sub, const uint16_t *
 int exl3_gemm(const uint16_t *xh, int rows, size_t ldx, const uint16_t *trellis, int in_tiles,
               int out_tiles, int K, int cb, int tn_offset, int tn_count, uint16_t *y_out,
               size_t ldy, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Prefill GEMM over rows that are sorted into groups (experts), each group
+ * multiplying its own tile columns of a stacked trellis: the segmented GEMM of
+ * the MoE prefill path (inner_mm_seg_mlx, ponyexl3/mlx/gemv_metal.py:1685-1741,
+ * called from EXL3SwitchGLU._prefill, ponyexl3/mlx/exl3_moe.py:684-768).
+ *   xh         fp16 [n_rows][ldx], rows of one group contiguous
+ *   group g multiplies tile columns [tn_base + g*group_tiles, + group_tiles)
+ *   group_tab  device int32 [n_row_blocks][4] = {group, first row, end row, 0}: row
+ *              blocks of at most block_rows (64, 128 or 256) rows that never span
+ *              two groups; first row == end row marks an unused entry (the
+ *              reference builds the same table on the device and sizes it for
+ *              the worst case, ponyexl3/mlx/exl3_moe.py:79-98, 722-723)
+ *   y_out      fp16 [n_rows][ldy] (ldy >= 16*group_tiles), same row order as xh
+ */
+int exl3_gemm_grouped(const uint16_t *xh, int n_rows, size_t ldx, const uint16_t *trellis,
+                      int in_tiles, int out_tiles, int K, int cb, int tn_base, int group_tiles,
+                      int n_groups, const int32_t *group_tab, int n_row_blocks, int block_rows,
+                      uint16_t *y_out, size_t ldy, void *stream);
 
 /* Scratch bytes exl3_gemm can use for this shape (0 when no tile would be split). */
 size_t exl3_gemm_workspace_bytes(int rows, int in_tiles, int tn_count);

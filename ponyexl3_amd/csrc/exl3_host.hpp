@@ -100,6 +100,14 @@ int launch_gemm(const uint16_t* xh, int rows, size_t ldx, const uint16_t* trelli
                 int out_tiles, int K, int cb, int tn_offset, int tn_count, uint16_t* y_out,
                 size_t ldy, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
+int launch_gemm_grouped(const uint16_t* xh, int n_rows, size_t ldx, const uint16_t* trellis,
+                        int in_tiles, int out_tiles, int K, int cb, int tn_base, int group_tiles,
+                        int n_groups, const int32_t* group_tab, int n_row_blocks, int block_rows,
+                        uint16_t* y_out, size_t ldy, hipStream_t stream);
+
+int launch_had_rows(const uint16_t* x, int rows, int n, const uint16_t* scale_rows, int post,
+                    uint16_t* out, hipStream_t stream);
+
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 // Integer tuning knob from the environment, clamped to [lo, hi].

@@ -73,9 +73,9 @@ __device__ __forceinline__ GemmWork gemm_work(int unit, int full_tiles, int spli
 template <int K, int CB, int MI>
 __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
     const uint32_t* __restrict__ trellis, const half_t* __restrict__ xh, half_t* __restrict__ y,
-    float* __restrict__ partial, int rows, size_t ldx, size_t ldy, int in_tiles, int out_tiles,
-    int tn_offset, int tn_count, int n_row_blocks, int full_tiles, int split,
-    int ksteps_per_split) {
+    float* __restrict__ partial, int rows_arg, size_t ldx, size_t ldy, int in_tiles, int out_tiles,
+    int tn_offset_arg, int tn_count_arg, int n_row_blocks, int full_tiles, int split,
+    int ksteps_per_split, const int4* __restrict__ group_tab, int group_tiles) {
     extern __shared__ __attribute__((aligned(16))) half_t smem[];
     constexpr int BM = 32 * MI;
     constexpr int STAGE_A = BM * 64, STAGE_B = kGemmStageB;
@@ -84,9 +84,34 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 2, wn = wave & 3;  // wave tile origin: rows wm*16*MI, columns wn*64
-    const GemmWork work = gemm_work(blockIdx.x, full_tiles, split, ksteps_per_split, in_tiles / 4);
-    const int g = work.tile / n_row_blocks;  // 256-column block inside the slice
-    const int m0 = (work.tile % n_row_blocks) * BM;
+    // Plain mode: work unit -> (column block g, row block) of one matrix, maybe one
+    // of several reduction ranges. Grouped mode (group_tab != NULL): the rows are
+    // sorted into groups (experts) that each multiply their own `group_tiles` tile
+    // columns; group_tab[b] = {group, first row, end row} of row block b (first ==
+    // end marks an unused entry), blockIdx.x = b * n_col_blocks + g, whole reduction.
+    GemmWork work;
+    int g, m0, rows, tn_offset, tn_count;
+    if (group_tab) {
+        const int n_col_blocks = (group_tiles + 15) >> 4;
+        const int4 t = group_tab[blockIdx.x / n_col_blocks];
+        if (t.y >= t.z) return;  // whole workgroup, before any barrier
+        work.tile = 0;
+        work.k_begin = 0;
+        work.k_end = in_tiles / 4;
+        work.partial_unit = -1;
+        g = blockIdx.x % n_col_blocks;
+        m0 = t.y;
+        rows = t.z;
+        tn_offset = tn_offset_arg + t.x * group_tiles;
+        tn_count = group_tiles;
+    } else {
+        work = gemm_work(blockIdx.x, full_tiles, split, ksteps_per_split, in_tiles / 4);
+        g = work.tile / n_row_blocks;  // 256-column block inside the slice
+        m0 = (work.tile % n_row_blocks) * BM;
+        rows = rows_arg;
+        tn_offset = tn_offset_arg;
+        tn_count = tn_count_arg;
+    }
     const int k_begin = work.k_begin, k_last = work.k_end - 1;
     const int nsteps = work.k_end - work.k_begin;
 
@@ -403,7 +428,7 @@ static int launch_gemm_mi(const GemmPlan& p, const uint16_t* xh, int rows, size_
     gemm_kernel<K, CB, MI><<<dim3(units), dim3(kGemmThreads), lds, stream>>>(
         reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<const half_t*>(xh),
         reinterpret_cast<half_t*>(y_out), partial, rows, ldx, ldy, in_tiles, out_tiles, tn_offset,
-        tn_count, p.n_row_blocks, p.full_tiles, p.split, p.ksteps_per_split);
+        tn_count, p.n_row_blocks, p.full_tiles, p.split, p.ksteps_per_split, nullptr, 0);
     if (int rc = launch_status()) return rc;
     if (p.split_tiles > 0) {
         gemm_fixup_kernel<MI><<<dim3((unsigned)p.split_tiles, 4 * MI), dim3(256), 0, stream>>>(
@@ -448,7 +473,70 @@ int launch_gemm(const uint16_t* xh, int rows, size_t ldx, const uint16_t* trelli
     });
 }
 
+template <int K, int CB, int MI>
+static int launch_gemm_grouped_mi(const uint16_t* xh, int n_rows, size_t ldx,
+                                  const uint16_t* trellis, int in_tiles, int out_tiles,
+                                  int tn_base, int group_tiles, const int32_t* group_tab,
+                                  int n_row_blocks, uint16_t* y_out, size_t ldy,
+                                  hipStream_t stream) {
+    constexpr size_t lds = (2 * (size_t)(32 * MI) * 64 + 2 * (size_t)kGemmStageB) * sizeof(half_t);
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_kernel<K, CB, MI>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return EXL3_E_LAUNCH;
+    const long long units = (long long)n_row_blocks * ((group_tiles + 15) / 16);
+    if (units > 0x7fffffffLL) return EXL3_E_BAD_SHAPE;
+    gemm_kernel<K, CB, MI><<<dim3((unsigned)units), dim3(kGemmThreads), lds, stream>>>(
+        reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<const half_t*>(xh),
+        reinterpret_cast<half_t*>(y_out), nullptr, n_rows, ldx, ldy, in_tiles, out_tiles, tn_base,
+        group_tiles, 1, 0, 1, in_tiles / 4, reinterpret_cast<const int4*>(group_tab), group_tiles);
+    return launch_status();
+}
+
+int launch_gemm_grouped(const uint16_t* xh, int n_rows, size_t ldx, const uint16_t* trellis,
+                        int in_tiles, int out_tiles, int K, int cb, int tn_base, int group_tiles,
+                        int n_groups, const int32_t* group_tab, int n_row_blocks, int block_rows,
+                        uint16_t* y_out, size_t ldy, hipStream_t stream) {
+    if (int rc = check_k_cb(K, cb)) return rc;
+    if (!xh || !trellis || !y_out || !group_tab) return EXL3_E_NULL_POINTER;
+    if (n_rows < 1 || in_tiles < 4 || in_tiles % 4 || tn_base < 0 || group_tiles < 8 ||
+        group_tiles % 8 || n_groups < 1 ||
+        (long long)tn_base + (long long)n_groups * group_tiles > out_tiles || n_row_blocks < 1 ||
+        ldx < (size_t)in_tiles * 16 || ldy < (size_t)group_tiles * 16 || ldx % 8 || ldy % 4)
+        return EXL3_E_BAD_SHAPE;
+    if (block_rows != 64 && block_rows != 128 && block_rows != 256) return EXL3_E_BAD_SHAPE;
+    if ((reinterpret_cast<uintptr_t>(xh) & 15) || (reinterpret_cast<uintptr_t>(y_out) & 7) ||
+        (reinterpret_cast<uintptr_t>(group_tab) & 15))
+        return EXL3_E_BAD_SHAPE;
+    if (ldx * 2 * 256 >= (1ull << 31)) return EXL3_E_BAD_SHAPE;
+    return dispatch_k_cb(K, cb, [&](auto k, auto c) {
+        if (block_rows == 64)
+            return launch_gemm_grouped_mi<k.value, c.value, 2>(xh, n_rows, ldx, trellis, in_tiles,
+                                                               out_tiles, tn_base, group_tiles,
+                                                               group_tab, n_row_blocks, y_out, ldy,
+                                                               stream);
+        if (block_rows == 128)
+            return launch_gemm_grouped_mi<k.value, c.value, 4>(xh, n_rows, ldx, trellis, in_tiles,
+                                                               out_tiles, tn_base, group_tiles,
+                                                               group_tab, n_row_blocks, y_out, ldy,
+                                                               stream);
+        return launch_gemm_grouped_mi<k.value, c.value, 8>(xh, n_rows, ldx, trellis, in_tiles,
+                                                           out_tiles, tn_base, group_tiles,
+                                                           group_tab, n_row_blocks, y_out, ldy,
+                                                           stream);
+    });
+}
+
 }  // namespace exl3
+
+EXL3_EXPORT int exl3_gemm_grouped(const uint16_t* xh, int n_rows, size_t ldx,
+                                  const uint16_t* trellis, int in_tiles, int out_tiles, int K,
+                                  int cb, int tn_base, int group_tiles, int n_groups,
+                                  const int32_t* group_tab, int n_row_blocks, int block_rows,
+                                  uint16_t* y_out, size_t ldy, void* stream) {
+    return exl3::launch_gemm_grouped(xh, n_rows, ldx, trellis, in_tiles, out_tiles, K, cb, tn_base,
+                                     group_tiles, n_groups, group_tab, n_row_blocks, block_rows,
+                                     y_out, ldy, exl3::as_stream(stream));
+}
 
 EXL3_EXPORT size_t exl3_gemm_workspace_bytes(int rows, int in_tiles, int tn_count) {
     if (rows < 1 || in_tiles < 4 || tn_count < 8) return 0;

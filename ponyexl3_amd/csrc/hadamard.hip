@@ -79,11 +79,12 @@ __device__ __forceinline__ void halfs_to_floats(uint4_t q, float (&v)[8]) {
 __global__ __launch_bounds__(256) void had_pre_wide_kernel(const half_t* __restrict__ x,
                                                            const half_t* __restrict__ suh,
                                                            half_t* __restrict__ xh, int n,
-                                                           int n_sub) {
+                                                           int n_sub, int scale_per_row) {
     const int lane = threadIdx.x & 63;
     const size_t rs = blockIdx.x;
     const half_t* xr = x + (rs / n_sub) * (size_t)n;
-    const half_t* sr = suh ? suh + (rs % n_sub) * (size_t)n : nullptr;
+    // scale vector: one per sub (stacked siblings) or one per row (rows sorted by expert)
+    const half_t* sr = suh ? suh + (scale_per_row ? rs : rs % n_sub) * (size_t)n : nullptr;
     half_t* orow = xh + rs * (size_t)n;
     for (int c = threadIdx.x * 8; c < n; c += 2048) {
         float v[8], sv[8];
@@ -110,8 +111,10 @@ __global__ __launch_bounds__(256) void had_pre_wide_kernel(const half_t* __restr
 __global__ __launch_bounds__(256) void had_post_wide_kernel(const half_t* __restrict__ y,
                                                             const half_t* __restrict__ svh,
                                                             const half_t* __restrict__ bias,
-                                                            half_t* out, int n) {
+                                                            half_t* out, int n,
+                                                            int scale_per_row) {
     const int lane = threadIdx.x & 63;
+    if (svh && scale_per_row) svh += (size_t)blockIdx.x * n;
     const half_t* yr = y + (size_t)blockIdx.x * n;
     half_t* orow = out + (size_t)blockIdx.x * n;
     for (int c = threadIdx.x * 8; c < n; c += 2048) {
@@ -254,7 +257,7 @@ int launch_had_pre(const uint16_t* x, int rows, int n, const uint16_t* suh, int 
         (!suh || aligned16(suh))) {
         had_pre_wide_kernel<<<dim3((unsigned)(rows * n_sub)), dim3(256), 0, stream>>>(
             reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(suh),
-            reinterpret_cast<half_t*>(xh), n, n_sub);
+            reinterpret_cast<half_t*>(xh), n, n_sub, 0);
         return launch_status();
     }
     had_pre_kernel<<<dim3((unsigned)grid), dim3(256), 0, stream>>>(
@@ -278,7 +281,7 @@ int launch_had_post(const void* y, int y_is_fp32, int n_sum, size_t sum_stride, 
     if (!y_is_fp32 && rows >= kWideMinRows && aligned16(y) && aligned16(out) &&
         (!svh || aligned16(svh)) && (!bias || aligned16(bias))) {
         had_post_wide_kernel<<<dim3((unsigned)rows), dim3(256), 0, stream>>>(
-            reinterpret_cast<const half_t*>(y), s, b, o, n);
+            reinterpret_cast<const half_t*>(y), s, b, o, n, 0);
         return launch_status();
     }
     if (y_is_fp32)
@@ -290,7 +293,30 @@ int launch_had_post(const void* y, int y_is_fp32, int n_sum, size_t sum_stride, 
     return launch_status();
 }
 
+// Per-row scale vectors (rows that belong to different experts): wide kernels only.
+int launch_had_rows(const uint16_t* x, int rows, int n, const uint16_t* scale_rows, int post,
+                    uint16_t* out, hipStream_t stream) {
+    if (!x || !out || !scale_rows) return EXL3_E_NULL_POINTER;
+    if (rows < 0 || n <= 0 || n % 128) return EXL3_E_BAD_SHAPE;
+    if (!aligned16(x) || !aligned16(out) || !aligned16(scale_rows)) return EXL3_E_BAD_SHAPE;
+    if (rows == 0) return EXL3_OK;
+    if (post)
+        had_post_wide_kernel<<<dim3((unsigned)rows), dim3(256), 0, stream>>>(
+            reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(scale_rows), nullptr,
+            reinterpret_cast<half_t*>(out), n, 1);
+    else
+        had_pre_wide_kernel<<<dim3((unsigned)rows), dim3(256), 0, stream>>>(
+            reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(scale_rows),
+            reinterpret_cast<half_t*>(out), n, 1, 1);
+    return launch_status();
+}
+
 }  // namespace exl3
+
+EXL3_EXPORT int exl3_had128_rows(const uint16_t* x, int rows, int n, const uint16_t* scale_rows,
+                                 int post, uint16_t* out, void* stream) {
+    return exl3::launch_had_rows(x, rows, n, scale_rows, post, out, exl3::as_stream(stream));
+}
 
 EXL3_EXPORT int exl3_had128_pre(const uint16_t* x, int rows, int n, const uint16_t* suh, int n_sub,
                                 uint16_t* xh, void* stream) {

@@ -80,6 +80,18 @@ class EXL3SwitchGLU(torch.nn.Module):
             activation=activation,
         )
 
+    # The sorted, segmented prefill path replaces the per-slot kernels once the
+    # experts see a few rows each (the reference switches at 9 tokens,
+    # ponyexl3/mlx/exl3_moe.py:770-787). Measured on 256 experts of 2048 x 512,
+    # top-8: the slot kernels cost ~4 us per token, the prefill path ~0.45 ms plus
+    # ~0.25 us per token, so they cross near 128 tokens = 4 rows per expert.
+    prefill_min_tokens = 24
+    prefill_min_rows_per_expert = 4.0
+
+    def _use_prefill(self, tokens: int, top_k: int) -> bool:
+        return (tokens >= self.prefill_min_tokens
+                and tokens * top_k >= self.prefill_min_rows_per_expert * self.num_experts)
+
     def forward(self, x: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
         if indices.dim() != 3:
             raise ValueError("indices must be (B, S, top_k)")
@@ -88,6 +100,8 @@ class EXL3SwitchGLU(torch.nn.Module):
         D = self.input_dims
         x2d = x.reshape(R, D).to(torch.float16).contiguous()
         idx = indices.reshape(R, kk).to(torch.int32).contiguous()
+        if self._use_prefill(R, kk):
+            return self._prefill(x2d, idx).reshape(B, S, kk, D)
         chunk = max(1, 4096 // kk)
         outs = []
         for r0 in range(0, R, chunk):
@@ -100,6 +114,44 @@ class EXL3SwitchGLU(torch.nn.Module):
             )
         y = outs[0] if len(outs) == 1 else torch.cat(outs, dim=0)
         return y.reshape(B, S, kk, D)
+
+    def _prefill(self, x2d: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
+        """Many tokens: sort the (token, slot) pairs by expert so that every expert's
+        weights are decoded once per block of its rows, rotate with per-row sign
+        vectors, run the segmented MFMA GEMM, finish per row, unsort
+        (``EXL3SwitchGLU._prefill``, ponyexl3/mlx/exl3_moe.py:684-768). No host
+        synchronisation: the block table is built on the device for the worst case."""
+        E, D, H = self.num_experts, self.input_dims, self.hidden_dims
+        R, kk = idx.shape
+        N = R * kk
+        flat = idx.reshape(-1).long().clamp_(0, E - 1)
+        order = torch.argsort(flat, stable=True)
+        sidx = flat[order]
+        tok = torch.div(order, kk, rounding_mode="floor")
+        per_expert = N / E
+        block_rows = 64 if per_expert <= 48 else 128 if per_expert <= 112 else 256
+        table = ops.segment_table(sidx, E, block_rows)
+        x_pairs = x2d[tok]
+        k, cb = self._k, self._cb
+        gt, dt = H // 16, D // 16
+        xg = ops.had128_rows(x_pairs, self._gu_suh[sidx, 0], post=False)
+        xu = ops.had128_rows(x_pairs, self._gu_suh[sidx, 1], post=False)
+        g = ops.gemm_grouped(xg, self._gu_trellis, k, cb, 0, gt, E, table, block_rows)
+        u = ops.gemm_grouped(xu, self._gu_trellis, k, cb, E * gt, gt, E, table, block_rows)
+        svh = self._gu_svh[sidx]
+        g = ops.had128_rows(g, svh[:, :H].contiguous(), post=True).float()
+        u = ops.had128_rows(u, svh[:, H:].contiguous(), post=True).float()
+        if self._activation == "gelu":
+            act = torch.nn.functional.gelu(g, approximate="tanh")
+        else:
+            act = torch.nn.functional.silu(g)
+        h = (act * u).to(torch.float16)
+        xd = ops.had128_rows(h, self._dn_suh[sidx], post=False)
+        y = ops.gemm_grouped(xd, self._dn_trellis, k, cb, 0, dt, E, table, block_rows)
+        y = ops.had128_rows(y, self._dn_svh[sidx], post=True)
+        out = torch.empty_like(y)
+        out[order] = y
+        return out.reshape(R, kk, D)
 
 
 def route_topk(logits: torch.Tensor, top_k: int, norm_topk_prob: bool = True):

@@ -376,6 +376,72 @@ def gemm_into(xh_ptr: int, rows: int, ldx: int, trellis, k: int, cb: int, tn_off
     _lib.check(rc, "exl3_gemm")
 
 
+def had128_rows(x2d: torch.Tensor, scale_rows: torch.Tensor, post: bool) -> torch.Tensor:
+    """Hadamard-128 with one scale vector per row: ``fp16(had(x * s))`` (``post``
+    False, ``_rows_prep``) or ``fp16(had(x) * s)`` (``post`` True, ``_rows_finish``;
+    ponyexl3/mlx/exl3_moe.py:105-136)."""
+    _half(x2d, "x")
+    _half(scale_rows, "scale_rows")
+    if x2d.dim() != 2 or scale_rows.shape != x2d.shape:
+        raise ValueError("x and scale_rows must both be (rows, n)")
+    rows, n = x2d.shape
+    if n % 128:
+        raise ValueError(f"feature dim {n} not divisible by 128")
+    out = torch.empty_like(x2d)
+    rc = _lib.load().exl3_had128_rows(_ptr(x2d), rows, n, _ptr(scale_rows), int(bool(post)),
+                                      _ptr(out), _stream())
+    _lib.check(rc, "exl3_had128_rows")
+    return out
+
+
+def segment_table(sorted_groups: torch.Tensor, n_groups: int, block_rows: int) -> torch.Tensor:
+    """Row-block table for ``gemm_grouped``: rows are sorted by group id; every block
+    of at most ``block_rows`` rows lies inside one group. Built with device-side
+    torch ops only (no host sync), sized for the worst case ``N // block_rows +
+    n_groups`` with unused entries marked empty, like the reference's table
+    (ponyexl3/mlx/exl3_moe.py:79-98). Returns int32 (n_blocks, 4) = {group, first
+    row, end row, 0}."""
+    n = sorted_groups.numel()
+    dev = sorted_groups.device
+    nb_max = n // block_rows + n_groups
+    cnt = torch.bincount(sorted_groups, minlength=n_groups)[:n_groups]
+    seg_end = torch.cumsum(cnt, 0)
+    seg_start = seg_end - cnt
+    nblk = (cnt + block_rows - 1) // block_rows
+    blk_end = torch.cumsum(nblk, 0)
+    blk_start = blk_end - nblk
+    b = torch.arange(nb_max, device=dev)
+    e = torch.searchsorted(blk_end, b, right=True).clamp_(max=n_groups - 1)
+    row0 = seg_start[e] + (b - blk_start[e]) * block_rows
+    end = seg_end[e]
+    row0 = torch.where(b < blk_end[-1], row0, end)
+    return torch.stack([e, row0, end, torch.zeros_like(e)], dim=1).to(torch.int32).contiguous()
+
+
+def gemm_grouped(xh, trellis, k: int, cb: int, tn_base: int, group_tiles: int, n_groups: int,
+                 table: torch.Tensor, block_rows: int):
+    """Segmented prefill GEMM: rows of ``xh`` (N, in) are sorted into groups, group g
+    multiplies tile columns ``tn_base + g*group_tiles ..`` (``inner_mm_seg_mlx``,
+    ponyexl3/mlx/gemv_metal.py:1685-1741). Returns (N, 16*group_tiles) fp16."""
+    in_tiles, out_tiles = _trellis_dims(trellis, k)
+    _half(xh, "xh")
+    if xh.dim() != 2 or xh.shape[1] != in_tiles * 16:
+        raise ValueError(f"xh must be (rows, {in_tiles * 16})")
+    if table.dtype != torch.int32 or table.dim() != 2 or table.shape[1] != 4:
+        raise ValueError("table must be int32 (n_blocks, 4)")
+    n = xh.shape[0]
+    y = torch.empty((n, group_tiles * 16), dtype=torch.float16, device=xh.device)
+    if n == 0:
+        return y
+    rc = _lib.load().exl3_gemm_grouped(
+        _ptr(xh), n, in_tiles * 16, _ptr(trellis), in_tiles, out_tiles, int(k), int(cb), int(tn_base),
+        int(group_tiles), int(n_groups), _ptr(table), table.shape[0], int(block_rows), _ptr(y),
+        group_tiles * 16, _stream(),
+    )
+    _lib.check(rc, "exl3_gemm_grouped")
+    return y
+
+
 def linear_forward(x2d, trellis, k, cb, suh=None, svh=None, bias=None, group_sub=None,
                    fused: bool = True, member_out=None):
     """Whole-layer forward on (rows, in) fp16 (``exl3_linear_forward``).

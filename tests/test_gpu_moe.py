@@ -73,6 +73,34 @@ def test_two_launch_and_five_launch_chains(cuda, oracle, tokens):
     assert rel_l2(y1.cpu().numpy(), y5.cpu().numpy()) <= TOL
 
 
+@pytest.mark.parametrize("tokens,act", [(40, "silu"), (200, "gelu")])
+def test_prefill_path_matches_oracle_and_slot_kernels(cuda, oracle, tokens, act):
+    """From 24 tokens on the pairs are sorted by expert and go through the segmented
+    GEMM. Experts with no token, one token and many tokens occur; checked against
+    the oracle chain and against the per-slot kernels on the same input."""
+    from ponyexl3_amd import EXL3SwitchGLU, ops
+
+    E, D, H, kk, k = 7, 256, 128, 2, 4
+    gate, up, down = _experts(E, D, H, k, False, 800)
+    moe = EXL3SwitchGLU.from_layers(gate, up, down, activation=act)
+    rng = np.random.default_rng(80 + tokens)
+    x = (rng.standard_normal((tokens, D)) * 0.5).astype(np.float16)
+    # skewed routing: expert 5 never chosen, expert 6 exactly once, the rest unevenly
+    p = np.array([0.45, 0.25, 0.15, 0.1, 0.05])
+    idx = np.stack([rng.choice(5, size=kk, replace=False, p=p) for _ in range(tokens)]).astype(np.int32)
+    idx[3, 1] = 6
+    xt, it = torch.from_numpy(x).to(cuda), torch.from_numpy(idx).to(cuda)
+    print(f"moe prefill tokens={tokens} act={act}", flush=True)
+    y = moe(xt.reshape(1, tokens, D), it.reshape(1, tokens, kk))[0]
+    assert tuple(y.shape) == (tokens, kk, D)
+    ref = _oracle_chain(oracle, gate, up, down, x, idx, act)
+    assert rel_l2(y.cpu().numpy(), ref) <= TOL
+    slots = torch.cat([ops.moe_forward(xt[r:r + 8], it[r:r + 8], moe._gu_trellis, moe._gu_suh, moe._gu_svh,
+                                       moe._dn_trellis, moe._dn_suh, moe._dn_svh, k, moe._cb,
+                                       0 if act == "silu" else 1) for r in range(0, tokens, 8)])
+    assert rel_l2(y.cpu().numpy(), slots.cpu().numpy()) <= TOL
+
+
 def test_moe_equals_linear_modules(cuda):
     """The stacked chain equals the same experts run as individual EXL3Linear
     modules (fused-vs-unfused, ponyexl3/tests/test_moe_activation.py:44-65)."""
