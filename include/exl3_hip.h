@@ -87,13 +87,19 @@ int exl3_had128_pre(const uint16_t *x, int rows, int n, const uint16_t *suh, int
  *   out         fp16 [rows][n]; may alias y when y is fp16
  */
 /*
- * Hadamard-128 with one scale vector per row (rows routed to different experts):
- *   post == 0: out = fp16(had128(x * scale_rows))   (_rows_prep, ponyexl3/mlx/exl3_moe.py:105-119)
- *   post != 0: out = fp16(had128(x) * scale_rows)   (_rows_finish, ponyexl3/mlx/exl3_moe.py:122-136)
- * x, scale_rows, out fp16 [rows][n], 16-byte aligned, n a multiple of 128.
+ * Hadamard-128 with one scale vector per row (rows routed to different experts),
+ * with the row gathers and the final scatter of the sorted MoE prefill folded in:
+ *   post == 0: out[o(r)] = fp16(had128(x[i(r)] * scale[s(r)]))  (_rows_prep,
+ *              ponyexl3/mlx/exl3_moe.py:105-119, with the x_pairs / suh gathers of :706-709)
+ *   post != 0: out[o(r)] = fp16(had128(x[i(r)]) * scale[s(r)])  (_rows_finish,
+ *              ponyexl3/mlx/exl3_moe.py:122-136, with the unsort of :768)
+ *   i = in_index, s = scale_index, o = out_index: device int32[rows], or NULL for
+ *   the identity; scale rows are scale_ld elements apart (a multiple of 8).
+ * x, out fp16 rows of n elements (n a multiple of 128); x, scale, out 16-byte aligned.
  */
-int exl3_had128_rows(const uint16_t *x, int rows, int n, const uint16_t *scale_rows, int post,
-                     uint16_t *out, void *stream);
+int exl3_had128_rows(const uint16_t *x, int rows, int n, const int32_t *in_index,
+                     const uint16_t *scale, const int32_t *scale_index, size_t scale_ld, int post,
+                     uint16_t *out, const int32_t *out_index, void *stream);
 
 int exl3_had128_post(const void *y, int y_is_fp32, int n_sum, size_t sum_stride, int rows, int n,
                      const uint16_t *svh, const uint16_t *bias, uint16_t *out, void *stream);

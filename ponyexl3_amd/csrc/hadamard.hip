@@ -38,6 +38,20 @@ __device__ __forceinline__ void wht128(float& a, float& b, int lane) {
     }
 }
 
+// Optional row gathers / scatter of the wide kernels: kernel row r reads input row
+// in_index[r], scale vector scale_index[r] (scale_ld elements apart) and writes
+// output row out_index[r]; a NULL table is the identity.
+struct RowMap {
+    int per_row;
+    const int32_t* in_index;
+    const int32_t* scale_index;
+    const int32_t* out_index;
+    size_t scale_ld;
+    __device__ size_t in_row(size_t r) const { return in_index ? (size_t)in_index[r] : r; }
+    __device__ size_t scale_row(size_t r) const { return scale_index ? (size_t)scale_index[r] : r; }
+    __device__ size_t out_row(size_t r) const { return out_index ? (size_t)out_index[r] : r; }
+};
+
 // v[j] = element 8*(lane & 15) + j of the lane group's block, unnormalised WHT in place.
 __device__ __forceinline__ void wht128_wide(float (&v)[8], int lane) {
 #pragma unroll
@@ -79,13 +93,16 @@ __device__ __forceinline__ void halfs_to_floats(uint4_t q, float (&v)[8]) {
 __global__ __launch_bounds__(256) void had_pre_wide_kernel(const half_t* __restrict__ x,
                                                            const half_t* __restrict__ suh,
                                                            half_t* __restrict__ xh, int n,
-                                                           int n_sub, int scale_per_row) {
+                                                           int n_sub, RowMap map) {
     const int lane = threadIdx.x & 63;
     const size_t rs = blockIdx.x;
-    const half_t* xr = x + (rs / n_sub) * (size_t)n;
-    // scale vector: one per sub (stacked siblings) or one per row (rows sorted by expert)
-    const half_t* sr = suh ? suh + (scale_per_row ? rs : rs % n_sub) * (size_t)n : nullptr;
-    half_t* orow = xh + rs * (size_t)n;
+    // source row and scale vector: (row, sub) product for stacked siblings, or
+    // per-row tables for rows that were sorted by expert
+    const half_t* xr = x + (map.per_row ? map.in_row(rs) : rs / n_sub) * (size_t)n;
+    const half_t* sr =
+        suh ? suh + (map.per_row ? map.scale_row(rs) * map.scale_ld : (rs % n_sub) * (size_t)n)
+            : nullptr;
+    half_t* orow = xh + map.out_row(rs) * (size_t)n;
     for (int c = threadIdx.x * 8; c < n; c += 2048) {
         float v[8], sv[8];
         halfs_to_floats(*reinterpret_cast<const uint4_t*>(xr + c), v);
@@ -111,12 +128,12 @@ __global__ __launch_bounds__(256) void had_pre_wide_kernel(const half_t* __restr
 __global__ __launch_bounds__(256) void had_post_wide_kernel(const half_t* __restrict__ y,
                                                             const half_t* __restrict__ svh,
                                                             const half_t* __restrict__ bias,
-                                                            half_t* out, int n,
-                                                            int scale_per_row) {
+                                                            half_t* out, int n, RowMap map) {
     const int lane = threadIdx.x & 63;
-    if (svh && scale_per_row) svh += (size_t)blockIdx.x * n;
-    const half_t* yr = y + (size_t)blockIdx.x * n;
-    half_t* orow = out + (size_t)blockIdx.x * n;
+    const size_t rs = blockIdx.x;
+    if (svh && map.per_row) svh += map.scale_row(rs) * map.scale_ld;
+    const half_t* yr = y + map.in_row(rs) * (size_t)n;
+    half_t* orow = out + map.out_row(rs) * (size_t)n;
     for (int c = threadIdx.x * 8; c < n; c += 2048) {
         float v[8], sv[8];
         halfs_to_floats(*reinterpret_cast<const uint4_t*>(yr + c), v);
@@ -257,7 +274,7 @@ int launch_had_pre(const uint16_t* x, int rows, int n, const uint16_t* suh, int 
         (!suh || aligned16(suh))) {
         had_pre_wide_kernel<<<dim3((unsigned)(rows * n_sub)), dim3(256), 0, stream>>>(
             reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(suh),
-            reinterpret_cast<half_t*>(xh), n, n_sub, 0);
+            reinterpret_cast<half_t*>(xh), n, n_sub, RowMap{});
         return launch_status();
     }
     had_pre_kernel<<<dim3((unsigned)grid), dim3(256), 0, stream>>>(
@@ -281,7 +298,7 @@ int launch_had_post(const void* y, int y_is_fp32, int n_sum, size_t sum_stride, 
     if (!y_is_fp32 && rows >= kWideMinRows && aligned16(y) && aligned16(out) &&
         (!svh || aligned16(svh)) && (!bias || aligned16(bias))) {
         had_post_wide_kernel<<<dim3((unsigned)rows), dim3(256), 0, stream>>>(
-            reinterpret_cast<const half_t*>(y), s, b, o, n, 0);
+            reinterpret_cast<const half_t*>(y), s, b, o, n, RowMap{});
         return launch_status();
     }
     if (y_is_fp32)
@@ -294,28 +311,33 @@ int launch_had_post(const void* y, int y_is_fp32, int n_sum, size_t sum_stride, 
 }
 
 // Per-row scale vectors (rows that belong to different experts): wide kernels only.
-int launch_had_rows(const uint16_t* x, int rows, int n, const uint16_t* scale_rows, int post,
-                    uint16_t* out, hipStream_t stream) {
-    if (!x || !out || !scale_rows) return EXL3_E_NULL_POINTER;
-    if (rows < 0 || n <= 0 || n % 128) return EXL3_E_BAD_SHAPE;
-    if (!aligned16(x) || !aligned16(out) || !aligned16(scale_rows)) return EXL3_E_BAD_SHAPE;
+int launch_had_rows(const uint16_t* x, int rows, int n, const int32_t* in_index,
+                    const uint16_t* scale, const int32_t* scale_index, size_t scale_ld, int post,
+                    uint16_t* out, const int32_t* out_index, hipStream_t stream) {
+    if (!x || !out || !scale) return EXL3_E_NULL_POINTER;
+    if (rows < 0 || n <= 0 || n % 128 || scale_ld % 8) return EXL3_E_BAD_SHAPE;
+    if (!aligned16(x) || !aligned16(out) || !aligned16(scale)) return EXL3_E_BAD_SHAPE;
     if (rows == 0) return EXL3_OK;
+    const RowMap map{1, in_index, scale_index, out_index, scale_ld};
     if (post)
         had_post_wide_kernel<<<dim3((unsigned)rows), dim3(256), 0, stream>>>(
-            reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(scale_rows), nullptr,
-            reinterpret_cast<half_t*>(out), n, 1);
+            reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(scale), nullptr,
+            reinterpret_cast<half_t*>(out), n, map);
     else
         had_pre_wide_kernel<<<dim3((unsigned)rows), dim3(256), 0, stream>>>(
-            reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(scale_rows),
-            reinterpret_cast<half_t*>(out), n, 1, 1);
+            reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(scale),
+            reinterpret_cast<half_t*>(out), n, 1, map);
     return launch_status();
 }
 
 }  // namespace exl3
 
-EXL3_EXPORT int exl3_had128_rows(const uint16_t* x, int rows, int n, const uint16_t* scale_rows,
-                                 int post, uint16_t* out, void* stream) {
-    return exl3::launch_had_rows(x, rows, n, scale_rows, post, out, exl3::as_stream(stream));
+EXL3_EXPORT int exl3_had128_rows(const uint16_t* x, int rows, int n, const int32_t* in_index,
+                                 const uint16_t* scale, const int32_t* scale_index,
+                                 size_t scale_ld, int post, uint16_t* out,
+                                 const int32_t* out_index, void* stream) {
+    return exl3::launch_had_rows(x, rows, n, in_index, scale, scale_index, scale_ld, post, out,
+                                 out_index, exl3::as_stream(stream));
 }
 
 EXL3_EXPORT int exl3_had128_pre(const uint16_t* x, int rows, int n, const uint16_t* suh, int n_sub,

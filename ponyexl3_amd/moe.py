@@ -83,8 +83,9 @@ class EXL3SwitchGLU(torch.nn.Module):
     # The sorted, segmented prefill path replaces the per-slot kernels once the
     # experts see a few rows each (the reference switches at 9 tokens,
     # ponyexl3/mlx/exl3_moe.py:770-787). Measured on 256 experts of 2048 x 512,
-    # top-8: the slot kernels cost ~4 us per token, the prefill path ~0.45 ms plus
-    # ~0.25 us per token, so they cross near 128 tokens = 4 rows per expert.
+    # top-8: the slot kernels cost ~4 us per token, the prefill path ~0.5 ms (every
+    # expert's weights are decoded once) plus ~0.15 us per token, so they cross near
+    # 128 tokens = 4 rows per expert.
     prefill_min_tokens = 24
     prefill_min_rows_per_expert = 4.0
 
@@ -131,27 +132,26 @@ class EXL3SwitchGLU(torch.nn.Module):
         per_expert = N / E
         block_rows = 64 if per_expert <= 48 else 128 if per_expert <= 112 else 256
         table = ops.segment_table(sidx, E, block_rows)
-        x_pairs = x2d[tok]
         k, cb = self._k, self._cb
         gt, dt = H // 16, D // 16
-        xg = ops.had128_rows(x_pairs, self._gu_suh[sidx, 0], post=False)
-        xu = ops.had128_rows(x_pairs, self._gu_suh[sidx, 1], post=False)
+        sidx32, tok32, order32 = sidx.int(), tok.int(), order.int()
+        # rotations read x through the token table and the signs through the expert table
+        xg = ops.had128_rows(x2d, self._gu_suh[:, 0], False, in_index=tok32, scale_index=sidx32)
+        xu = ops.had128_rows(x2d, self._gu_suh[:, 1], False, in_index=tok32, scale_index=sidx32)
         g = ops.gemm_grouped(xg, self._gu_trellis, k, cb, 0, gt, E, table, block_rows)
         u = ops.gemm_grouped(xu, self._gu_trellis, k, cb, E * gt, gt, E, table, block_rows)
-        svh = self._gu_svh[sidx]
-        g = ops.had128_rows(g, svh[:, :H].contiguous(), post=True).float()
-        u = ops.had128_rows(u, svh[:, H:].contiguous(), post=True).float()
+        g = ops.had128_rows(g, self._gu_svh[:, :H], True, scale_index=sidx32).float()
+        u = ops.had128_rows(u, self._gu_svh[:, H:], True, scale_index=sidx32).float()
         if self._activation == "gelu":
             act = torch.nn.functional.gelu(g, approximate="tanh")
         else:
             act = torch.nn.functional.silu(g)
         h = (act * u).to(torch.float16)
-        xd = ops.had128_rows(h, self._dn_suh[sidx], post=False)
+        xd = ops.had128_rows(h, self._dn_suh, False, scale_index=sidx32)
         y = ops.gemm_grouped(xd, self._dn_trellis, k, cb, 0, dt, E, table, block_rows)
-        y = ops.had128_rows(y, self._dn_svh[sidx], post=True)
-        out = torch.empty_like(y)
-        out[order] = y
-        return out.reshape(R, kk, D)
+        # finish and scatter back to (token, slot) order in one pass
+        y = ops.had128_rows(y, self._dn_svh, True, scale_index=sidx32, out_index=order32)
+        return y.reshape(R, kk, D)
 
 
 def route_topk(logits: torch.Tensor, top_k: int, norm_topk_prob: bool = True):

@@ -376,20 +376,33 @@ def gemm_into(xh_ptr: int, rows: int, ldx: int, trellis, k: int, cb: int, tn_off
     _lib.check(rc, "exl3_gemm")
 
 
-def had128_rows(x2d: torch.Tensor, scale_rows: torch.Tensor, post: bool) -> torch.Tensor:
+def had128_rows(x2d: torch.Tensor, scale: torch.Tensor, post: bool, *, rows: int | None = None,
+                in_index=None, scale_index=None, out_index=None) -> torch.Tensor:
     """Hadamard-128 with one scale vector per row: ``fp16(had(x * s))`` (``post``
     False, ``_rows_prep``) or ``fp16(had(x) * s)`` (``post`` True, ``_rows_finish``;
-    ponyexl3/mlx/exl3_moe.py:105-136)."""
+    ponyexl3/mlx/exl3_moe.py:105-136). Output row r is computed from input row
+    ``in_index[r]`` and scale row ``scale_index[r]`` and stored at ``out_index[r]``
+    (int32 device tensors; None = identity). ``scale`` is a 2D view whose rows may
+    be strided (e.g. ``gu_suh[:, 0]``)."""
     _half(x2d, "x")
-    _half(scale_rows, "scale_rows")
-    if x2d.dim() != 2 or scale_rows.shape != x2d.shape:
-        raise ValueError("x and scale_rows must both be (rows, n)")
-    rows, n = x2d.shape
+    if not isinstance(scale, torch.Tensor) or not scale.is_cuda or scale.dtype != torch.float16:
+        raise ValueError("scale must be an fp16 tensor on the GPU")
+    if x2d.dim() != 2 or scale.dim() != 2 or scale.shape[1] != x2d.shape[1] or scale.stride(1) != 1:
+        raise ValueError("x and scale must be (rows, n) with unit inner stride")
+    n = x2d.shape[1]
+    if rows is None:
+        rows = x2d.shape[0] if in_index is None else in_index.numel()
+    for name, t in (("in_index", in_index), ("scale_index", scale_index), ("out_index", out_index)):
+        if t is not None:
+            _check_cuda(t, name)
+            if t.dtype != torch.int32 or t.numel() != rows:
+                raise ValueError(f"{name} must be int32 with one entry per row")
     if n % 128:
         raise ValueError(f"feature dim {n} not divisible by 128")
-    out = torch.empty_like(x2d)
-    rc = _lib.load().exl3_had128_rows(_ptr(x2d), rows, n, _ptr(scale_rows), int(bool(post)),
-                                      _ptr(out), _stream())
+    out = torch.empty((rows, n), dtype=torch.float16, device=x2d.device)
+    rc = _lib.load().exl3_had128_rows(
+        _ptr(x2d), rows, n, _ptr(in_index), _ptr(scale), _ptr(scale_index), scale.stride(0),
+        int(bool(post)), _ptr(out), _ptr(out_index), _stream())
     _lib.check(rc, "exl3_had128_rows")
     return out
 
