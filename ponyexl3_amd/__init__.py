@@ -22,6 +22,7 @@ __all__ = [
     "FusedEXL3Group",
     "FusedEXL3Sibling",
     "EXL3SwitchGLU",
+    "EXL3MoEBlock",
     "fusable",
     "reconstruct_inner",
     "reconstruct_public_weights",
@@ -38,7 +39,7 @@ def __getattr__(name):
         from . import fused
 
         return getattr(fused, name)
-    if name in ("EXL3SwitchGLU", "route_topk", "combine_experts"):
+    if name in ("EXL3SwitchGLU", "EXL3MoEBlock", "route_topk", "combine_experts"):
         from . import moe
 
         return getattr(moe, name)

@@ -167,3 +167,39 @@ def route_topk(logits: torch.Tensor, top_k: int, norm_topk_prob: bool = True):
 def combine_experts(y: torch.Tensor, scores: torch.Tensor) -> torch.Tensor:
     """(…, kk, D) x (…, kk) -> (…, D) (ponyexl3/mlx/exl3_moe.py:838-839)."""
     return (y * scores[..., None].to(y.dtype)).sum(dim=-2)
+
+
+class EXL3MoEBlock(torch.nn.Module):
+    """Router + routed experts + weighted sum (``EXL3MoEBlock``,
+    ponyexl3/mlx/exl3_moe.py:790-839). With ``shared_gate`` the shared expert is
+    stacked as the LAST expert of ``switch`` and always selected, its routing
+    weight being ``sigmoid(shared_gate(x))``; the router only ranks the others.
+    ``x (..., D) -> (..., D)``."""
+
+    def __init__(self, gate: torch.nn.Module, shared_gate: torch.nn.Module | None,
+                 switch: EXL3SwitchGLU, top_k: int, norm_topk_prob: bool = True):
+        super().__init__()
+        self.gate = gate
+        self.shared_expert_gate = shared_gate
+        self.switch_mlp = switch
+        self.top_k = int(top_k)
+        self.norm_topk_prob = bool(norm_topk_prob)
+        self._shared_idx = switch.num_experts - 1
+
+    def route(self, x: torch.Tensor):
+        inds, scores = route_topk(self.gate(x), self.top_k, self.norm_topk_prob)
+        scores = scores.to(x.dtype)
+        if self.shared_expert_gate is not None:
+            shared_w = torch.sigmoid(self.shared_expert_gate(x)).to(x.dtype)
+            shared = torch.full(inds.shape[:-1] + (1,), self._shared_idx, dtype=inds.dtype,
+                                device=inds.device)
+            inds = torch.cat([inds, shared], dim=-1)
+            scores = torch.cat([scores, shared_w], dim=-1)
+        return inds, scores
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        lead = tuple(x.shape[:-1])
+        x3 = x.reshape(1, -1, x.shape[-1])
+        inds, scores = self.route(x3)
+        y = self.switch_mlp(x3, inds)
+        return combine_experts(y, scores).reshape(lead + (x.shape[-1],))

@@ -183,3 +183,32 @@ def test_errors(cuda):
     with pytest.raises(ValueError):
         EXL3SwitchGLU(gu_trellis=zi(8, 8, 64), gu_suh=z(1, 2, 128), gu_svh=z(1, 256), dn_trellis=zi(8, 8, 64),
                       dn_suh=z(1, 128), dn_svh=z(1, 128), k=4, cb=0)
+
+
+def test_moe_block_with_shared_expert(cuda, oracle):
+    """Router (softmax, top-k, renormalise), the shared expert stacked last with a
+    sigmoid gate, weighted sum: against the same composition over the oracle chain
+    (ponyexl3/mlx/exl3_moe.py:790-839)."""
+    from ponyexl3_amd import EXL3MoEBlock, EXL3SwitchGLU
+
+    E, D, H, kk = 5, 256, 128, 2  # 4 routed experts + the shared one
+    gate, up, down = _experts(E, D, H, 4, True, 950)
+    switch = EXL3SwitchGLU.from_layers(gate, up, down)
+    g = torch.Generator().manual_seed(2)
+    router = torch.nn.Linear(D, E - 1, bias=False)
+    shared_gate = torch.nn.Linear(D, 1, bias=False)
+    with torch.no_grad():
+        router.weight.copy_(torch.randn((E - 1, D), generator=g) * 0.2)
+        shared_gate.weight.copy_(torch.randn((1, D), generator=g) * 0.2)
+    block = EXL3MoEBlock(router.half().to(cuda), shared_gate.half().to(cuda), switch, kk).to(cuda)
+    x = (torch.randn((3, D), generator=g) * 0.5).to(torch.float16)
+    with torch.no_grad():
+        y = block(x.to(cuda)).float().cpu().numpy()
+        inds, scores = block.route(x.to(cuda).reshape(1, 3, D))
+    assert y.shape == (3, D)
+    inds, scores = inds[0].cpu().numpy(), scores[0].float().cpu().numpy()
+    assert inds.shape == (3, kk + 1) and (inds[:, -1] == E - 1).all() and (inds[:, :kk] < E - 1).all()
+    np.testing.assert_allclose(scores[:, :kk].sum(axis=1), 1.0, atol=2e-3)
+    per_expert = _oracle_chain(oracle, gate, up, down, x.numpy(), inds.astype(np.int32), "silu")
+    ref = (per_expert.astype(np.float32) * scores[..., None]).sum(axis=1)
+    assert rel_l2(y, ref) <= 2 * TOL  # fp16 products and sum over three experts on top of the chain
