@@ -30,6 +30,26 @@ def test_gemm_matches_oracle(cuda, oracle, rows, k, cb):
     assert rel_l2(y, ref) < 5e-4  # one fp16 rounding of the result
 
 
+@pytest.mark.parametrize("k", [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("cb", [0, 1, 2])
+def test_identity_activations_reproduce_the_decoded_weights_bit_for_bit(cuda, oracle, k, cb):
+    """x = I makes every output the sum of one weight and zeros, which fp32 MFMA
+    accumulation and the single fp16 cast keep exact: the GEMM's in-kernel decode,
+    LDS layout and fragment mapping against the oracle's decoded weights, every bit
+    width and codebook, 64-, 128- and 256-row blocks."""
+    from ponyexl3_amd import ops
+
+    rng = np.random.default_rng(600 + 10 * k + cb)
+    tr_np = rng.integers(0, 65536, size=(24, 24, 16 * k), dtype=np.uint16)  # 384 -> 384
+    tr = ops.as_trellis_tensor(tr_np, cuda)
+    w = oracle.decode_trellis(tr_np, k, cb).view(np.uint16)
+    eye = torch.eye(384, dtype=torch.float16, device=cuda)
+    print(f"gemm identity k={k} cb={cb}", flush=True)
+    for rows in (384, 100, 40):  # MI = 8, 4, 2
+        y = ops.inner_gemm(eye[:rows].contiguous(), tr, k, cb).cpu().numpy().view(np.uint16)
+        np.testing.assert_array_equal(y, w[:rows])
+
+
 def test_gemm_column_slice(cuda, oracle):
     from ponyexl3_amd import ops
 

@@ -115,3 +115,21 @@ def test_errors(cuda):
         ops.inner_gem_fused(torch.zeros((9, 1, 128), dtype=torch.float16, device=cuda), tr, 4, 0)
     with pytest.raises(ValueError):
         ops.inner_gem_fused(torch.zeros((1, 2, 128), dtype=torch.float16, device=cuda), tr, 4, 0)
+
+
+@pytest.mark.parametrize("k,cb", [(1, 0), (2, 1), (3, 0), (4, 0), (4, 1), (4, 2), (5, 1), (6, 0), (7, 1), (8, 0)])
+def test_one_hot_activations_reproduce_the_decoded_weights_exactly(cuda, oracle, k, cb):
+    """A one-hot activation row selects one row of W: the fp32 result must equal the
+    oracle's decoded fp16 weight exactly, for every row count of the kernel."""
+    from ponyexl3_amd import ops
+
+    rng = np.random.default_rng(700 + 10 * k + cb)
+    tr_np = rng.integers(0, 65536, size=(16, 16, 16 * k), dtype=np.uint16)  # 256 -> 256
+    tr = ops.as_trellis_tensor(tr_np, cuda)
+    w = oracle.decode_trellis(tr_np, k, cb).astype(np.float32)
+    for rows in (1, 2, 3, 4, 8):
+        pick = rng.permutation(256)[:rows]
+        xh = torch.zeros((rows, 1, 256), dtype=torch.float16, device=cuda)
+        xh[torch.arange(rows), 0, torch.from_numpy(pick).to(cuda)] = 1.0
+        y = ops.inner_gem_fused(xh, tr, k, cb).cpu().numpy()
+        np.testing.assert_array_equal(y, w[pick])
