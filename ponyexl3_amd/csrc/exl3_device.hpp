@@ -158,10 +158,13 @@ __device__ __forceinline__ uint32_t lane_codeword(const LaneWords<K>& lw) {
     constexpr int wi = (end - 1) / 32;
     constexpr int sh = 32 * (wi + 1) - end;
     if constexpr (sh + 16 <= 32) {
-        return (lw.w[wi] >> sh) & 0xFFFFu;
+        return (lw.w[wi] >> sh) & 0xFFFFu;  // one v_bfe_u32 (v_and / v_lshrrev at the ends)
     } else {
-        const uint64_t pair = ((uint64_t)lw.w[wi - 1] << 32) | lw.w[wi];
-        return (uint32_t)(pair >> sh) & 0xFFFFu;
+        // The window straddles two dwords. All straddling windows of one dword pair
+        // share the same 16-bit funnel shift (one v_alignbit_b32, merged by common
+        // subexpression elimination), after which each is one v_bfe_u32.
+        const uint32_t mid = __builtin_amdgcn_alignbit(lw.w[wi - 1], lw.w[wi], 16);
+        return (mid >> (sh - 16)) & 0xFFFFu;
     }
 }
 
