@@ -59,6 +59,23 @@ int exl3_decode_full(const uint16_t *trellis, int in_tiles, int out_tiles, int K
                      int tn_offset, int tn_count, uint16_t *w_out, void *stream);
 
 /*
+ * Stacked-expert trellis -> contiguous per-expert matrices: tile column t goes to
+ * expert t / tiles_per_e. Replaces decode_full_eg_mlx
+ * (ponyexl3/mlx/gemv_metal.py:746-774). out_tiles must be a multiple of tiles_per_e.
+ *   w_out   fp16 [out_tiles/tiles_per_e][16*in_tiles][16*tiles_per_e]
+ */
+int exl3_decode_full_eg(const uint16_t *trellis, int in_tiles, int out_tiles, int K, int cb,
+                        int tiles_per_e, uint16_t *w_out, void *stream);
+
+/*
+ * Trellis -> fp16 W_inner transposed, for a slice of tile columns. Replaces
+ * decode_full_t_mlx (ponyexl3/mlx/gemv_metal.py:841-866).
+ *   w_out_t fp16 [16*tn_count][16*in_tiles] row-major
+ */
+int exl3_decode_full_t(const uint16_t *trellis, int in_tiles, int out_tiles, int K, int cb,
+                       int tn_offset, int tn_count, uint16_t *w_out_t, void *stream);
+
+/*
  * Input-side Hadamard-128 with per-channel multipliers, fp32 butterflies:
  *   xh[r][s][:] = fp16( H128/sqrt(128) applied per 128-block to (x[r][:] * suh[s][:]) )
  * Replaces EXL3LayerRuntime.prepare_xh (ponyexl3/mlx/layer_state.py:133-136),

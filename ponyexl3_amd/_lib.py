@@ -33,6 +33,8 @@ PROTOTYPES = {
     "exl3_status_string": (ctypes.c_char_p, [_i]),
     "exl3_gemv_max_rows": (_i, []),
     "exl3_decode_full": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _vp]),
+    "exl3_decode_full_eg": (_i, [_vp, _i, _i, _i, _i, _i, _vp, _vp]),
+    "exl3_decode_full_t": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _vp]),
     "exl3_had128_pre": (_i, [_vp, _i, _i, _vp, _i, _vp, _vp]),
     "exl3_had128_post": (_i, [_vp, _i, _i, _sz, _i, _i, _vp, _vp, _vp, _vp]),
     "exl3_gemv": (_i, [_vp, _i, _i, _vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _sz, _vp]),

@@ -137,6 +137,40 @@ def decode_full(trellis, k: int, cb: int, tn_offset: int = 0, tn_count: int | No
     return w
 
 
+def decode_full_eg(trellis, k: int, cb: int, *, tiles_per_e: int):
+    """Stacked-expert trellis -> contiguous (E, in, 16*tiles_per_e) fp16
+    (``decode_full_eg_mlx``, ponyexl3/mlx/gemv_metal.py:746-774)."""
+    in_tiles, out_tiles = _trellis_dims(trellis, k)
+    if tiles_per_e < 1 or out_tiles % tiles_per_e != 0:
+        raise ValueError("out_tiles not divisible by tiles_per_e")
+    w = torch.empty((out_tiles // tiles_per_e, in_tiles * 16, tiles_per_e * 16), dtype=torch.float16,
+                    device=trellis.device)
+    if w.numel() == 0:
+        return w
+    rc = _lib.load().exl3_decode_full_eg(
+        _ptr(trellis), in_tiles, out_tiles, int(k), int(cb), int(tiles_per_e), _ptr(w), _stream())
+    _lib.check(rc, "exl3_decode_full_eg")
+    return w
+
+
+def decode_full_t(trellis, k: int, cb: int, tn_offset: int = 0, tn_count: int | None = None):
+    """Trellis -> fp16 W^T (16*tn_count, in) (``decode_full_t_mlx``,
+    ponyexl3/mlx/gemv_metal.py:841-866)."""
+    in_tiles, out_tiles = _trellis_dims(trellis, k)
+    if tn_count is None:
+        tn_count = out_tiles - tn_offset
+    if tn_offset < 0 or tn_count < 0 or tn_offset + tn_count > out_tiles:
+        raise ValueError("slice exceeds output features")
+    w = torch.empty((tn_count * 16, in_tiles * 16), dtype=torch.float16, device=trellis.device)
+    if w.numel() == 0:
+        return w
+    rc = _lib.load().exl3_decode_full_t(
+        _ptr(trellis), in_tiles, out_tiles, int(k), int(cb), int(tn_offset), int(tn_count),
+        _ptr(w), _stream())
+    _lib.check(rc, "exl3_decode_full_t")
+    return w
+
+
 def reconstruct_inner(trellis, k: int, cb: int, n_offset: int = 0, n_count: int | None = None):
     """Inner weight W (in, n_count) fp16 for a 128-aligned column range
     (``reconstruct_inner``, ponyexl3/ref/reconstruct.py:13-23; the reference

@@ -54,6 +54,12 @@ def test_argument_errors_before_launch(lib):
     assert lib.exl3_decode_full(p, 1, 1, 4, 3, 0, 1, p, None) == _lib.EXL3_E_BAD_CODEBOOK
     assert lib.exl3_decode_full(None, 1, 1, 4, 0, 0, 1, p, None) == _lib.EXL3_E_NULL_POINTER
     assert lib.exl3_decode_full(p, 1, 1, 4, 0, 1, 1, p, None) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_decode_full_eg(p, 1, 6, 4, 0, 4, p, None) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_decode_full_eg(p, 1, 6, 4, 0, 0, p, None) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_decode_full_eg(p, 1, 6, 0, 0, 3, p, None) == _lib.EXL3_E_BAD_K
+    assert lib.exl3_decode_full_t(p, 1, 1, 4, 0, 1, 1, p, None) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_decode_full_t(p, 1, 1, 4, 0, 0, 1, None, None) == _lib.EXL3_E_NULL_POINTER
+    assert lib.exl3_decode_full_t(p, 0, 1, 4, 0, 0, 1, p, None) == _lib.EXL3_OK  # empty: no launch
     assert lib.exl3_had128_pre(p, 1, 100, None, 1, p, None) == _lib.EXL3_E_BAD_SHAPE
     assert lib.exl3_had128_post(p, 0, 2, 0, 1, 128, None, None, p, None) == _lib.EXL3_E_BAD_SHAPE
     assert lib.exl3_gemv(p, 9, 1, p, 8, 8, 4, 0, None, None, 1, p, p, 1 << 20, None) == _lib.EXL3_E_BAD_SHAPE

@@ -94,3 +94,43 @@ def test_reconstruct_public_weights(cuda, oracle):
     assert float((y - y_pub).norm() / y_pub.norm()) < 5e-3
     with pytest.raises(ValueError):
         ops.reconstruct_inner(tr, 3, int(layer.codebook_mode), n_offset=64)
+
+
+@pytest.mark.parametrize("k", range(1, 9))
+@pytest.mark.parametrize("cb", [0, 1, 2])
+def test_transposed_and_expert_grouped_layouts_bit_exact(cuda, oracle, k, cb):
+    """The (out, in) and (E, in, out_e) layouts hold exactly the weights of the
+    row-major decode (decode_full_t_mlx / decode_full_eg_mlx,
+    ponyexl3/mlx/gemv_metal.py:746-866); 11 tile rows and 21 / 12 tile columns
+    leave partly filled wavefronts in both kernels."""
+    from ponyexl3_amd import ops
+
+    rng = np.random.default_rng(900 + 10 * k + cb)
+    tr = rng.integers(0, 65536, size=(11, 12, 16 * k), dtype=np.uint16)
+    full = oracle.decode_trellis(tr, k, cb).view(np.uint16)  # (176, 192)
+    trt = ops.as_trellis_tensor(tr, cuda)
+    print(f"layouts k={k} cb={cb}", flush=True)
+    wt = ops.decode_full_t(trt, k, cb).cpu().numpy().view(np.uint16)
+    np.testing.assert_array_equal(wt, full.T)
+    for off, cnt in ((5, 3), (0, 1), (11, 1), (2, 9)):
+        wt = ops.decode_full_t(trt, k, cb, tn_offset=off, tn_count=cnt).cpu().numpy().view(np.uint16)
+        assert wt.shape == (16 * cnt, 176)
+        np.testing.assert_array_equal(wt, full[:, 16 * off:16 * (off + cnt)].T)
+    for tpe in (1, 3, 4, 12):
+        eg = ops.decode_full_eg(trt, k, cb, tiles_per_e=tpe).cpu().numpy().view(np.uint16)
+        assert eg.shape == (12 // tpe, 176, 16 * tpe)
+        for e in range(12 // tpe):
+            np.testing.assert_array_equal(eg[e], full[:, 16 * tpe * e:16 * tpe * (e + 1)])
+
+
+def test_layout_variant_errors(cuda):
+    from ponyexl3_amd import ops
+
+    tr = torch.zeros((2, 6, 64), dtype=torch.int16, device=cuda)
+    with pytest.raises(ValueError):
+        ops.decode_full_eg(tr, 4, 0, tiles_per_e=4)  # 6 tile columns do not split into fours
+    with pytest.raises(ValueError):
+        ops.decode_full_eg(tr, 4, 0, tiles_per_e=0)
+    with pytest.raises(ValueError):
+        ops.decode_full_t(tr, 4, 0, tn_offset=5, tn_count=2)
+    assert tuple(ops.decode_full_t(tr, 4, 0, tn_offset=6, tn_count=0).shape) == (0, 32)
