@@ -265,6 +265,37 @@ int exl3_moe_forward(const uint16_t *x, int tokens, const int32_t *indices, int 
 
 size_t exl3_moe_workspace_bytes(int tokens, int top_k, int D, int H);
 
+/*
+ * Encoder side: tail-biting Viterbi search over the bitshift trellis, one 16x16
+ * tile (256 fp32 targets in kernel order) per workgroup. Replaces
+ * quantize_tiles_mlx (ponyexl3/convert/metal_search.py:63-196, 254-303) and
+ * follows its arithmetic (fp16 path costs, fp32 fma, warm-up pass + pinned pass),
+ * so the same path is chosen; the exact float64 search
+ * (ponyexl3/convert/reference_search.py:59-87) is the quality yardstick.
+ * K must be in 2..8 (the reference rejects K = 1 too): EXL3_E_BAD_K otherwise.
+ *   tiles     fp32 [n_tiles][256]
+ *   q_tiles   fp32 [n_tiles][256]   decoded value of the chosen codeword
+ *   indices   u16  [n_tiles][256]   full 16-bit codewords; indices & (2^K - 1) are
+ *                                   the symbols exl3_pack_trellis takes
+ *   workspace backpointer slots, exl3_quantize_slot_bytes(K) each. At least one
+ *             slot is required (EXL3_E_WORKSPACE); exl3_quantize_workspace_bytes()
+ *             is what keeps every CU busy; more than that is not used. A tile
+ *             batch larger than the slot count is walked by the same launch.
+ */
+size_t exl3_quantize_slot_bytes(int K);
+size_t exl3_quantize_workspace_bytes(int n_tiles, int K);
+int exl3_quantize_tiles(const float *tiles, int n_tiles, int K, int cb, float *q_tiles,
+                        uint16_t *indices, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * K-bit symbols (low K bits of each u16) -> packed tiles, bit-exact with
+ * pack_trellis (ponyexl3/ref/trellis.py:13-49, 144-150) and pack_trellis_mlx
+ * (ponyexl3/convert/mlx_trellis.py:66-84). K in 1..8.
+ *   encoded u16 [n_tiles][256]   packed u16 [n_tiles][16*K] (4-byte aligned)
+ */
+int exl3_pack_trellis(const uint16_t *encoded, long long n_tiles, int K, uint16_t *packed,
+                      void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -35,6 +35,23 @@
  *   exl3o_moe_expert       composition of pinned parts; the reference has no CPU
  *                          twin for the MoE chain (only Metal kernels), so the
  *                          chain as a whole is "parity unpinned" beyond that.
+ *   exl3o_quantize_tile_exact
+ *                          exact Viterbi over the bitshift trellis
+ *                          (convert/reference_search.py). Pinned by what the
+ *                          mathematics fixes: brute force over every closed path
+ *                          of a short trellis, recovery of exactly representable
+ *                          tiles, the tail-biting closure, pack -> unpack round
+ *                          trip of its states (the reference's own assertions,
+ *                          tests/test_convert_metal.py:25-86).
+ *   exl3o_quantize_tiles_search
+ *                          the production search kernel's arithmetic
+ *                          (convert/metal_search.py:63-196: compressed states,
+ *                          fp16 cost storage, warm-up pass + one pinned pass).
+ *                          Pinned by the same assertions plus the reference's
+ *                          quality bound against the exact search (mse <= 1.10 x).
+ *                          Its bit-for-bit agreement with the Metal kernel itself
+ *                          cannot be checked here (no Metal): "parity unpinned"
+ *                          for the exact path chosen among near-ties.
  */
 #include <math.h>
 #include <stdint.h>
@@ -407,6 +424,178 @@ EXL3O_API int exl3o_linear_forward_bs1(const uint16_t *trellis, int in_tiles, in
     for (int c = 0; c < out; c++) y[c] = f2h(yh[c]);
     free(xf); free(xh); free(yf); free(yh); free(table); free(part);
     return 0;
+}
+
+/* ---------------------------------------------------------------- search */
+
+static float *decode_lut_f32(int cb) {
+    float *lut = (float *)malloc(65536 * sizeof(float));
+    if (lut)
+        for (uint32_t c = 0; c < 65536u; c++) lut[c] = h2f(exl3o_decode_cw(c, cb));
+    return lut;
+}
+
+/* convert/reference_search.py:32-56 _forward: one Viterbi pass over 2^16 states
+ * with float64 path costs. s' = ((s << K) | fresh) & 0xFFFF, so the predecessors
+ * of s' are (s' >> K) | (j << (16-K)), j = 0..2^K-1; ties keep the lowest j
+ * (numpy argmin). init_state < 0: free start. n_steps = 256 in the reference; the
+ * parameter only exists so a short trellis can be brute-forced in the tests. */
+static int viterbi_forward(const float *w, int n_steps, int k, const float *lut, int init_state,
+                           uint16_t *back, double *cost, double *next) {
+    const int kk = 1 << k;
+    for (int s = 0; s < 65536; s++) cost[s] = init_state < 0 ? 0.0 : 1e30;
+    if (init_state >= 0) cost[init_state] = 0.0;
+    for (int t = 0; t < n_steps; t++) {
+        const double wt = (double)w[t];
+#pragma omp parallel for schedule(static)
+        for (int s = 0; s < 65536; s++) {
+            uint32_t best_p = (uint32_t)s >> k;
+            double best = cost[best_p];
+            for (int j = 1; j < kk; j++) {
+                const uint32_t p = ((uint32_t)s >> k) | ((uint32_t)j << (16 - k));
+                if (cost[p] < best) {
+                    best = cost[p];
+                    best_p = p;
+                }
+            }
+            back[(size_t)t * 65536 + s] = (uint16_t)best_p;
+            const double d = (double)lut[s] - wt;
+            next[s] = best + d * d;
+        }
+        memcpy(cost, next, 65536 * sizeof(double));
+    }
+    int fin = 0;
+    for (int s = 1; s < 65536; s++)
+        if (cost[s] < cost[fin]) fin = s;
+    return fin;
+}
+
+/* convert/reference_search.py:59-87 quantize_tile_reference: free pass, then up
+ * to max_pins passes pinned to the previous pass's last state until the path
+ * closes (pre-state of step 0 == states[n-1] == pin). */
+EXL3O_API int exl3o_quantize_tile_exact(const float *w, int n_steps, int k, int cb, int max_pins,
+                                        uint16_t *states, float *decoded) {
+    if (k < 1 || k > 8 || cb < 0 || cb > 2 || n_steps < 1) return -1;
+    float *lut = decode_lut_f32(cb);
+    uint16_t *back = (uint16_t *)malloc((size_t)n_steps * 65536 * sizeof(uint16_t));
+    double *cost = (double *)malloc(2 * 65536 * sizeof(double));
+    if (!lut || !back || !cost) {
+        free(lut); free(back); free(cost);
+        return -2;
+    }
+    int pin = -1;
+    for (int pass = 0; pass <= max_pins; pass++) {
+        int s = viterbi_forward(w, n_steps, k, lut, pin, back, cost, cost + 65536);
+        for (int t = n_steps - 1; t >= 0; t--) {
+            states[t] = (uint16_t)s;
+            s = back[(size_t)t * 65536 + s];
+        }
+        const int last = states[n_steps - 1];
+        if (pass > 0 && s == pin && last == pin) break;
+        pin = last;
+    }
+    for (int t = 0; t < n_steps; t++) decoded[t] = lut[states[t]];
+    free(lut); free(back); free(cost);
+    return 0;
+}
+
+/* convert/metal_search.py:63-196, one tile per call of the inner body.
+ * Compressed state e = the newest 16-K bits; the candidate codeword for
+ * (fresh, e) is (fresh << (16-K)) | e with predecessor cw >> K. Costs are kept
+ * as fp16 between steps (:128,153), arithmetic is fp32 with one fma (:147),
+ * clamped to 65504; ties keep the lowest fresh (strict <, :123,149). Pass 0
+ * starts at position 128, runs once around and backtracks to the state before
+ * position 0 (:176-190); pass 1 starts at 0 pinned to it and must end in it. */
+EXL3O_API int exl3o_quantize_tiles_search(const float *tiles, int n_tiles, int k, int cb,
+                                          float *q_tiles, uint16_t *indices) {
+    if (k < 2 || k > 8 || cb < 0 || cb > 2 || n_tiles < 0) return -1;
+    const int kr = 16 - k, edges = 1 << kr, kk = 1 << k;
+    const float H_INF = 65504.0f;
+    float *lut = decode_lut_f32(cb);
+    if (!lut) return -2;
+    int rc = 0;
+#pragma omp parallel for schedule(dynamic)
+    for (int tile = 0; tile < n_tiles; tile++) {
+        uint16_t *edge_ptr = (uint16_t *)malloc((size_t)256 * edges * sizeof(uint16_t));
+        uint16_t *costs = (uint16_t *)malloc((size_t)2 * edges * sizeof(uint16_t));
+        if (!edge_ptr || !costs) {
+            rc = -2;
+            free(edge_ptr); free(costs);
+            continue;
+        }
+        const float *in_tile = tiles + (size_t)tile * 256;
+        float *out_tile = q_tiles + (size_t)tile * 256;
+        uint16_t *out_idx = indices + (size_t)tile * 256;
+        uint32_t pin = 0;
+        int pinned = 0;
+        for (int pass = 0; pass < 2; pass++) {
+            int curr = 0;
+            const int roll = pass == 0 ? 128 : 0;
+            for (int step = 0; step < 256; step++) {
+                const int ri = (step + roll) & 255;
+                const int prev_buf = curr;
+                if (step > 0) curr = 1 - curr;
+                const float target = in_tile[ri];
+                for (int e = 0; e < edges; e++) {
+                    float best = H_INF;
+                    uint32_t best_pred = 0;
+                    for (int fresh = 0; fresh < kk; fresh++) {
+                        const uint32_t cw = ((uint32_t)fresh << kr) | (uint32_t)e;
+                        const uint32_t pred = cw >> k;
+                        float err;
+                        if (step == 0) {
+                            if (pinned && pred != pin) {
+                                err = H_INF;
+                            } else {
+                                const float dh = lut[cw] - target;
+                                err = dh * dh;
+                                if (err > H_INF) err = H_INF;
+                            }
+                        } else {
+                            const float dh = lut[cw] - target;
+                            err = fmaf(dh, dh, h2f(costs[(size_t)prev_buf * edges + pred]));
+                            if (err > H_INF) err = H_INF;
+                        }
+                        if (err < best) {
+                            best = err;
+                            best_pred = pred;
+                        }
+                    }
+                    costs[(size_t)curr * edges + e] = f2h(best);
+                    if (pass == 1 || ri < 128) edge_ptr[(size_t)ri * edges + e] = (uint16_t)best_pred;
+                }
+            }
+            uint32_t edge = pin;
+            if (pass == 0) {
+                float best = H_INF;
+                edge = 0;
+                for (int e = 0; e < edges; e++) {
+                    const float v = h2f(costs[(size_t)curr * edges + e]);
+                    if (v < best) {
+                        best = v;
+                        edge = (uint32_t)e;
+                    }
+                }
+            }
+            for (int step_i = 255; step_i >= 0; step_i--) {
+                const int ri = (step_i + roll) & 255;
+                const uint32_t prev = edge_ptr[(size_t)ri * edges + edge];
+                const uint32_t state = ((prev << k) | edge) & 0xFFFFu;
+                edge = prev;
+                if (pass == 1) {
+                    out_idx[ri] = (uint16_t)state;
+                    out_tile[ri] = lut[state];
+                } else if (ri == 0) {
+                    break;
+                }
+            }
+            pin = edge;
+            pinned = 1;
+        }
+        free(edge_ptr); free(costs);
+    }
+    free(lut);
+    return rc;
 }
 
 EXL3O_API int exl3o_num_threads(void) {

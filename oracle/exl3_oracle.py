@@ -59,6 +59,8 @@ def lib() -> ctypes.CDLL:
         L.exl3o_half_to_float.argtypes = [_u16p, _f32p, ctypes.c_size_t]
         L.exl3o_float_to_half.argtypes = [_f32p, _u16p, ctypes.c_size_t]
         L.exl3o_double_to_half.argtypes = [_f64p, _u16p, ctypes.c_size_t]
+        L.exl3o_quantize_tile_exact.argtypes = [_f32p] + [ctypes.c_int] * 4 + [_u16p, _f32p]
+        L.exl3o_quantize_tiles_search.argtypes = [_f32p] + [ctypes.c_int] * 3 + [_f32p, _u16p]
         L.exl3o_num_threads.restype = ctypes.c_int
         L.exl3o_set_num_threads.argtypes = [ctypes.c_int]
         _lib = L
@@ -286,6 +288,41 @@ def moe_experts_forward(experts, x, indices, k, cb, activation="silu"):
             h = glu(g, u, activation)
             out[t, s] = linear_forward(*e["down"][:1], k, cb, e["down"][1], e["down"][2], h)[0]
     return out
+
+
+def quantize_tile_exact(w: np.ndarray, k: int, cb: int, max_pins: int = 4):
+    """Exact Viterbi, float64 path costs (``quantize_tile_reference``,
+    ponyexl3/convert/reference_search.py:59-87). w: (n,) fp32 in kernel order, n = 256
+    for a tile (shorter trellises are for brute-force checks). Returns (states u16,
+    decoded fp32)."""
+    w = np.ascontiguousarray(w, dtype=np.float32).reshape(-1)
+    states = np.empty(w.size, dtype=np.uint16)
+    decoded = np.empty(w.size, dtype=np.float32)
+    rc = lib().exl3o_quantize_tile_exact(w.ctypes.data_as(_f32p), w.size, int(k), int(cb), int(max_pins),
+                                         _p16(states), decoded.ctypes.data_as(_f32p))
+    if rc:
+        raise ValueError(f"bad arguments (K={k}, cb={cb})")
+    return states, decoded
+
+
+def quantize_tiles_search(tiles: np.ndarray, k: int, cb: int):
+    """The production search's arithmetic (``quantize_tiles_mlx``,
+    ponyexl3/convert/metal_search.py:63-196, 254-303). tiles: (N, 256) fp32 in kernel
+    order. Returns (q_tiles fp32 (N, 256), full 16-bit codewords u16 (N, 256))."""
+    if not 2 <= int(k) <= 8:
+        raise ValueError("trellis search supports K in [2, 8]")
+    tiles = np.ascontiguousarray(tiles, dtype=np.float32)
+    if tiles.ndim == 1:
+        tiles = tiles.reshape(1, 256)
+    if tiles.ndim != 2 or tiles.shape[1] != 256:
+        raise ValueError(f"expected tiles shape (N, 256), got {tiles.shape}")
+    q = np.empty_like(tiles)
+    idx = np.empty(tiles.shape, dtype=np.uint16)
+    rc = lib().exl3o_quantize_tiles_search(tiles.ctypes.data_as(_f32p), tiles.shape[0], int(k), int(cb),
+                                           q.ctypes.data_as(_f32p), _p16(idx))
+    if rc:
+        raise ValueError(f"bad arguments (K={k}, cb={cb})")
+    return q, idx
 
 
 def num_threads() -> int:

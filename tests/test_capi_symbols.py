@@ -54,6 +54,15 @@ def test_argument_errors_before_launch(lib):
     assert lib.exl3_decode_full(p, 1, 1, 4, 3, 0, 1, p, None) == _lib.EXL3_E_BAD_CODEBOOK
     assert lib.exl3_decode_full(None, 1, 1, 4, 0, 0, 1, p, None) == _lib.EXL3_E_NULL_POINTER
     assert lib.exl3_decode_full(p, 1, 1, 4, 0, 1, 1, p, None) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_quantize_tiles(p, 1, 1, 0, p, p, p, 1 << 30, None) == _lib.EXL3_E_BAD_K
+    assert lib.exl3_quantize_tiles(p, 1, 4, 7, p, p, p, 1 << 30, None) == _lib.EXL3_E_BAD_CODEBOOK
+    assert lib.exl3_quantize_tiles(p, 1, 4, 0, p, p, None, 0, None) == _lib.EXL3_E_NULL_POINTER
+    assert lib.exl3_quantize_tiles(p, 1, 4, 0, p, p, p, 100, None) == _lib.EXL3_E_WORKSPACE
+    assert lib.exl3_quantize_tiles(p, 0, 4, 0, p, p, p, 0, None) == _lib.EXL3_OK  # empty: no launch
+    assert lib.exl3_quantize_slot_bytes(4) == 256 * 4096 * 2 and lib.exl3_quantize_slot_bytes(1) == 0
+    assert lib.exl3_pack_trellis(p, 1, 0, p, None) == _lib.EXL3_E_BAD_K
+    assert lib.exl3_pack_trellis(p, 1, 4, None, None) == _lib.EXL3_E_NULL_POINTER
+    assert lib.exl3_pack_trellis(p, 0, 4, p, None) == _lib.EXL3_OK
     assert lib.exl3_decode_full_eg(p, 1, 6, 4, 0, 4, p, None) == _lib.EXL3_E_BAD_SHAPE
     assert lib.exl3_decode_full_eg(p, 1, 6, 4, 0, 0, p, None) == _lib.EXL3_E_BAD_SHAPE
     assert lib.exl3_decode_full_eg(p, 1, 6, 0, 0, 3, p, None) == _lib.EXL3_E_BAD_K
