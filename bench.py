@@ -268,6 +268,7 @@ def main():
         extras.update(bench_config1(dev))
         extras.update(bench_prefill(dev, layers[0], xs))
         extras.update(bench_moe(dev))
+        extras.update(bench_encoder(dev))
     if args.sweep:
         extras.update(bench_sweep(dev, layers[0]))
 
@@ -432,6 +433,36 @@ def bench_prefill(dev, layer, xs):
                              "library_fp16_gemm_TFLOPs_gate_up_shape": round(lib_tf, 1),
                              "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "bound": "mfma",
                              "kernel": "gemm_kernel<K=4, cb=3INST>", "per_linear": per}}
+
+
+def bench_encoder(dev):
+    """Encoder side: tail-biting trellis search over 4096 tiles of N(0, 1.24^2)
+    targets (a 1024 x 1024 matrix) at K = 4, MCG, plus the symbol packer. Every step
+    of the search evaluates all 65536 codewords, 2 x 256 steps per tile; the kernel
+    spends five VALU instructions per evaluation."""
+    import torch
+
+    from ponyexl3_amd import search
+
+    n, k = 4096, 4
+    gen = torch.Generator(device=dev).manual_seed(50_004)
+    tiles = torch.randn((n, 256), device=dev, generator=gen) * 1.24371088
+    search.quantize_tiles(tiles[:64], k, 1)
+    keep = {}
+
+    def run():
+        keep["q"], keep["idx"] = search.quantize_tiles(tiles, k, 1)
+
+    ms = _time_ms(run, reps=3, warm=1)
+    mse = float(((keep["q"] - tiles) ** 2).mean())
+    evals = n * 2 * 256 * 65536
+    sym = keep["idx"] & ((1 << k) - 1)
+    pack_ms = _time_ms(lambda: search.pack_trellis(sym, k), reps=10, warm=2)
+    return {"encoder": {"workload": f"{n} tiles, K={k}, MCG", "ms": round(ms, 2),
+                        "tiles_per_s": round(n / ms * 1e3), "Mweights_per_s": round(n * 256 / ms / 1e3, 1),
+                        "T_evals_per_s": round(evals / ms / 1e9, 2),
+                        "T_valu_lane_ops_per_s": round(5 * evals / ms / 1e9, 1),
+                        "mse": round(mse, 5), "pack_trellis_us": round(pack_ms * 1e3, 1)}}
 
 
 def bench_moe(dev):

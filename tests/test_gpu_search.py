@@ -17,7 +17,7 @@ def _tiles(seed, n, scale=1.24371088):
 
 
 @pytest.mark.parametrize("k,cb", [(2, MCG), (3, MCG), (4, DEFAULT), (4, MCG), (4, MUL1), (5, DEFAULT),
-                                  (6, MCG), (7, MUL1), (8, MCG)])
+                                  (6, MCG), (7, MUL1), (7, MCG), (8, MCG), (8, DEFAULT)])
 def test_same_path_as_the_oracle_search(cuda, oracle, k, cb):
     """Integer outputs: bit-exact. The first tile of each case uses the seed and
     scale of the reference's quality test."""
