@@ -266,6 +266,29 @@ int exl3_moe_forward(const uint16_t *x, int tokens, const int32_t *indices, int 
 size_t exl3_moe_workspace_bytes(int tokens, int top_k, int D, int H);
 
 /*
+ * MoE prefill glue, one launch each.
+ * exl3_moe_sort: stable counting sort of the (token, slot) pairs by expert plus the
+ * row-block table exl3_gemm_grouped takes. Replaces the argsort / segment-table
+ * host code of EXL3SwitchGLU._prefill (ponyexl3/mlx/exl3_moe.py:79-98, 700-716).
+ *   indices i32 [n_pairs] expert per pair (pair = token*top_k + slot; clamped)
+ *   order, tok, sidx  i32 [n_pairs], by sorted position: pair index, token, expert
+ *   table   i32 [table_len][4] = {expert, first row, end row, 0}, 16-byte aligned,
+ *           table_len >= n_pairs / block_rows + n_experts; unused entries are empty
+ * n_experts <= 1024 (EXL3_E_UNSUPPORTED above that).
+ * exl3_moe_glu_rows: per sorted row r with expert e = sidx[r]:
+ *   xh_dn[r] = fp16(had(fp16(act(G) * U) * dn_suh[e])), G = fp16(had(g[r]) * gu_svh[e][:H]),
+ *   U likewise from u and gu_svh[e][H:]; activation 0 = SiLU, 1 = tanh-GELU. Replaces
+ *   _rows_finish x2, the GLU and _rows_prep (ponyexl3/mlx/exl3_moe.py:105-136, 62-75).
+ *   g, u, xh_dn fp16 [n_rows][H]; gu_svh fp16 [E][2*H]; dn_suh fp16 [E][H]
+ */
+int exl3_moe_sort(const int32_t *indices, int n_pairs, int top_k, int n_experts, int block_rows,
+                  int32_t *order, int32_t *tok, int32_t *sidx, int32_t *table, int table_len,
+                  void *stream);
+int exl3_moe_glu_rows(const uint16_t *g, const uint16_t *u, int n_rows, int H, const int32_t *sidx,
+                      const uint16_t *gu_svh, const uint16_t *dn_suh, int n_experts,
+                      int activation, uint16_t *xh_dn, void *stream);
+
+/*
  * Encoder side: tail-biting Viterbi search over the bitshift trellis, one 16x16
  * tile (256 fp32 targets in kernel order) per workgroup. Replaces
  * quantize_tiles_mlx (ponyexl3/convert/metal_search.py:63-196, 254-303) and

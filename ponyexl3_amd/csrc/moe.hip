@@ -366,6 +366,145 @@ static MoeWorkspace moe_workspace(int tokens, int top_k, int D, int H) {
     return w;
 }
 
+// ---------------------------------------------------------------------------
+// Prefill glue: sort the (token, slot) pairs by expert and build the row-block
+// table of the segmented GEMM in ONE launch of one workgroup (the pair counts are
+// small: tokens * top_k), and finish gate/up + GLU + down rotation per sorted row.
+
+constexpr int kSortThreads = 1024;
+constexpr int kSortMaxExperts = 1024;
+
+// Stable counting sort by expert id. Outputs, all indexed by sorted position:
+//   order[pos] = pair index (token * top_k + slot), tok[pos] = token,
+//   sidx[pos] = expert; table[b] = {expert, first row, end row of the expert, 0}
+// for every block of block_rows rows, unused entries {E-1, N, N, 0} (empty).
+__global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
+    const int* __restrict__ indices, int n_pairs, int top_k, int E, int block_rows,
+    int* __restrict__ order, int* __restrict__ tok, int* __restrict__ sidx,
+    int4* __restrict__ table, int table_len) {
+    __shared__ int count[kSortMaxExperts];  // pairs per expert, later the scatter cursor
+    __shared__ unsigned short wave_count[kSortThreads / 64][kSortMaxExperts];  // <= 64 each
+    __shared__ int scan_tmp[2][kSortThreads / 64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int e = tid; e < E; e += kSortThreads) count[e] = 0;
+    for (int i = tid; i < (kSortThreads / 64) * kSortMaxExperts; i += kSortThreads)
+        (&wave_count[0][0])[i] = 0;
+    __syncthreads();
+    for (int i = tid; i < n_pairs; i += kSortThreads) atomicAdd(&count[clamp_expert(indices[i], E)], 1);
+    __syncthreads();
+
+    // exclusive scans over the experts (E <= 1024 = one value per thread): rows and blocks
+    const int c = tid < E ? count[tid] : 0;
+    const int nb = (c + block_rows - 1) / block_rows;
+    int inc_rows = c, inc_blk = nb;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int r = __shfl_up(inc_rows, off, kWave), b = __shfl_up(inc_blk, off, kWave);
+        if (lane >= off) {
+            inc_rows += r;
+            inc_blk += b;
+        }
+    }
+    if (lane == 63) {
+        scan_tmp[0][wave] = inc_rows;
+        scan_tmp[1][wave] = inc_blk;
+    }
+    __syncthreads();
+    int base_rows = 0, base_blk = 0, total_blk = 0;
+    for (int w = 0; w < kSortThreads / 64; w++) {
+        if (w < wave) {
+            base_rows += scan_tmp[0][w];
+            base_blk += scan_tmp[1][w];
+        }
+        total_blk += scan_tmp[1][w];
+    }
+    const int row0 = base_rows + inc_rows - c;  // first sorted row of expert tid
+    const int blk0 = base_blk + inc_blk - nb;
+    __syncthreads();
+    if (tid < E) {
+        count[tid] = row0;  // scatter cursor
+        for (int b = 0; b < nb && blk0 + b < table_len; b++)
+            table[blk0 + b] = int4{tid, row0 + b * block_rows, row0 + c, 0};
+    }
+    for (int b = total_blk + tid; b < table_len; b += kSortThreads)
+        table[b] = int4{E - 1, n_pairs, n_pairs, 0};
+    __syncthreads();
+
+    // stable scatter, 1024 pairs at a time in pair order: rank inside the wave by
+    // matching expert ids bit by bit, then across the waves of the chunk
+    int ebits = 0;
+    while ((1 << ebits) < E) ebits++;
+    for (int i0 = 0; i0 < n_pairs; i0 += kSortThreads) {
+        const int i = i0 + tid;
+        const bool valid = i < n_pairs;
+        const int e = valid ? clamp_expert(indices[i], E) : 0;
+        unsigned long long same = __ballot(valid);
+        for (int b = 0; b < ebits; b++) {
+            const unsigned long long m = __ballot(valid && ((e >> b) & 1));
+            same &= ((e >> b) & 1) ? m : ~m;
+        }
+        const int rank = __popcll(same & ((1ull << lane) - 1ull));
+        if (valid && rank == 0) wave_count[wave][e] = (unsigned short)__popcll(same);
+        __syncthreads();
+        if (valid) {
+            int pos = count[e] + rank;
+            for (int w = 0; w < wave; w++) pos += wave_count[w][e];
+            order[pos] = i;
+            tok[pos] = i / top_k;
+            sidx[pos] = e;
+        }
+        __syncthreads();
+        for (int ee = tid; ee < E; ee += kSortThreads) {
+            int add = 0;
+#pragma unroll
+            for (int w = 0; w < kSortThreads / 64; w++) {
+                add += wave_count[w][ee];
+                wave_count[w][ee] = 0;
+            }
+            count[ee] += add;
+        }
+        __syncthreads();
+    }
+}
+
+// One wave per (sorted row, 128-block of H): post-Hadamard + svh of the gate and up
+// GEMM outputs, GLU, and the input rotation (dn_suh) of the down projection; the
+// same steps and casts as moe_glu_kernel, on fp16 GEMM outputs.
+__global__ __launch_bounds__(256) void moe_glu_rows_kernel(
+    const half_t* __restrict__ g, const half_t* __restrict__ u, int n_rows, int H,
+    const int* __restrict__ sidx, const half_t* __restrict__ gu_svh,
+    const half_t* __restrict__ dn_suh, int E, int activation, half_t* __restrict__ xh_dn) {
+    const int lane = threadIdx.x & 63;
+    const int hblocks = H >> 7;
+    const long long wave_id = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (wave_id >= (long long)n_rows * hblocks) return;
+    const int blk = (int)(wave_id % hblocks);
+    const size_t r = (size_t)(wave_id / hblocks);
+    const int e = clamp_expert(sidx[r], E);
+    const size_t off = r * H + blk * 128 + 2 * lane;
+    float v[2][2];
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+        const half2_t in = *reinterpret_cast<const half2_t*>((p ? u : g) + off);
+        float a = (float)in.x, b = (float)in.y;
+        wht128_lanes(a, b, lane);
+        const half2_t sv = *reinterpret_cast<const half2_t*>(gu_svh + (size_t)e * 2 * H + p * H +
+                                                             blk * 128 + 2 * lane);
+        v[p][0] = (float)(half_t)(a * kHadScaleF * (float)sv.x);
+        v[p][1] = (float)(half_t)(b * kHadScaleF * (float)sv.y);
+    }
+    const float h0 = (float)(half_t)glu_act(v[0][0], v[1][0], activation);
+    const float h1 = (float)(half_t)glu_act(v[0][1], v[1][1], activation);
+    const half2_t ds =
+        *reinterpret_cast<const half2_t*>(dn_suh + (size_t)e * H + blk * 128 + 2 * lane);
+    float a = h0 * (float)ds.x, b = h1 * (float)ds.y;
+    wht128_lanes(a, b, lane);
+    half2_t o;
+    o.x = (half_t)(a * kHadScaleF);
+    o.y = (half_t)(b * kHadScaleF);
+    *reinterpret_cast<half2_t*>(xh_dn + off) = o;
+}
+
 }  // namespace exl3
 
 EXL3_EXPORT size_t exl3_moe_workspace_bytes(int tokens, int top_k, int D, int H) {
@@ -460,4 +599,39 @@ EXL3_EXPORT int exl3_moe_forward(const uint16_t* x, int tokens, const int32_t* i
             num_experts);
         return launch_status();
     }
+}
+
+EXL3_EXPORT int exl3_moe_sort(const int32_t* indices, int n_pairs, int top_k, int n_experts,
+                              int block_rows, int32_t* order, int32_t* tok, int32_t* sidx,
+                              int32_t* table, int table_len, void* stream) {
+    using namespace exl3;
+    if (!indices || !order || !tok || !sidx || !table) return EXL3_E_NULL_POINTER;
+    if (n_pairs < 1 || top_k < 1 || n_experts < 1 || block_rows < 1 ||
+        table_len < n_pairs / block_rows + n_experts)
+        return EXL3_E_BAD_SHAPE;
+    if (n_experts > kSortMaxExperts) return EXL3_E_UNSUPPORTED;
+    if (reinterpret_cast<uintptr_t>(table) & 15) return EXL3_E_BAD_SHAPE;
+    moe_sort_kernel<<<dim3(1), dim3(kSortThreads), 0, as_stream(stream)>>>(
+        indices, n_pairs, top_k, n_experts, block_rows, order, tok, sidx,
+        reinterpret_cast<int4*>(table), table_len);
+    return launch_status();
+}
+
+EXL3_EXPORT int exl3_moe_glu_rows(const uint16_t* g, const uint16_t* u, int n_rows, int H,
+                                  const int32_t* sidx, const uint16_t* gu_svh,
+                                  const uint16_t* dn_suh, int n_experts, int activation,
+                                  uint16_t* xh_dn, void* stream) {
+    using namespace exl3;
+    if (!g || !u || !sidx || !gu_svh || !dn_suh || !xh_dn) return EXL3_E_NULL_POINTER;
+    if (n_rows < 0 || H < 128 || H % 128 || n_experts < 1) return EXL3_E_BAD_SHAPE;
+    if (activation < 0 || activation > 1) return EXL3_E_UNSUPPORTED;
+    if (n_rows == 0) return EXL3_OK;
+    const long long waves = (long long)n_rows * (H / 128);
+    const long long grid = (waves + 3) / 4;
+    if (grid > 0x7FFFFFFFLL) return EXL3_E_BAD_SHAPE;
+    moe_glu_rows_kernel<<<dim3((unsigned)grid), dim3(256), 0, as_stream(stream)>>>(
+        reinterpret_cast<const half_t*>(g), reinterpret_cast<const half_t*>(u), n_rows, H, sidx,
+        reinterpret_cast<const half_t*>(gu_svh), reinterpret_cast<const half_t*>(dn_suh), n_experts,
+        activation, reinterpret_cast<half_t*>(xh_dn));
+    return launch_status();
 }

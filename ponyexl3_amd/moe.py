@@ -125,29 +125,27 @@ class EXL3SwitchGLU(torch.nn.Module):
         E, D, H = self.num_experts, self.input_dims, self.hidden_dims
         R, kk = idx.shape
         N = R * kk
-        flat = idx.reshape(-1).long().clamp_(0, E - 1)
-        order = torch.argsort(flat, stable=True)
-        sidx = flat[order]
-        tok = torch.div(order, kk, rounding_mode="floor")
         per_expert = N / E
         block_rows = 64 if per_expert <= 48 else 128 if per_expert <= 112 else 256
-        table = ops.segment_table(sidx, E, block_rows)
+        if E <= ops.MOE_SORT_MAX_EXPERTS:
+            order32, tok32, sidx32, table = ops.moe_sort(idx, E, block_rows)  # one launch
+        else:
+            flat = idx.reshape(-1).long().clamp_(0, E - 1)
+            order = torch.argsort(flat, stable=True)
+            sidx = flat[order]
+            table = ops.segment_table(sidx, E, block_rows)
+            sidx32, order32 = sidx.int(), order.int()
+            tok32 = torch.div(order, kk, rounding_mode="floor").int()
         k, cb = self._k, self._cb
         gt, dt = H // 16, D // 16
-        sidx32, tok32, order32 = sidx.int(), tok.int(), order.int()
         # rotations read x through the token table and the signs through the expert table
         xg = ops.had128_rows(x2d, self._gu_suh[:, 0], False, in_index=tok32, scale_index=sidx32)
         xu = ops.had128_rows(x2d, self._gu_suh[:, 1], False, in_index=tok32, scale_index=sidx32)
         g = ops.gemm_grouped(xg, self._gu_trellis, k, cb, 0, gt, E, table, block_rows)
         u = ops.gemm_grouped(xu, self._gu_trellis, k, cb, E * gt, gt, E, table, block_rows)
-        g = ops.had128_rows(g, self._gu_svh[:, :H], True, scale_index=sidx32).float()
-        u = ops.had128_rows(u, self._gu_svh[:, H:], True, scale_index=sidx32).float()
-        if self._activation == "gelu":
-            act = torch.nn.functional.gelu(g, approximate="tanh")
-        else:
-            act = torch.nn.functional.silu(g)
-        h = (act * u).to(torch.float16)
-        xd = ops.had128_rows(h, self._dn_suh, False, scale_index=sidx32)
+        # finish gate and up, GLU, rotate for the down projection: one launch
+        xd = ops.moe_glu_rows(g, u, sidx32, self._gu_svh, self._dn_suh,
+                              _MOE_ACTIVATIONS[self._activation])
         y = ops.gemm_grouped(xd, self._dn_trellis, k, cb, 0, dt, E, table, block_rows)
         # finish and scatter back to (token, slot) order in one pass
         y = ops.had128_rows(y, self._dn_svh, True, scale_index=sidx32, out_index=order32)

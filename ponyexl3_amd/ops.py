@@ -465,6 +465,53 @@ def segment_table(sorted_groups: torch.Tensor, n_groups: int, block_rows: int) -
     return torch.stack([e, row0, end, torch.zeros_like(e)], dim=1).to(torch.int32).contiguous()
 
 
+MOE_SORT_MAX_EXPERTS = 1024
+
+
+def moe_sort(indices: torch.Tensor, n_experts: int, block_rows: int):
+    """Stable sort of the (token, slot) pairs of ``indices`` (T, top_k) int32 by
+    expert, with the row-block table of :func:`gemm_grouped`, in one launch
+    (``exl3_moe_sort``; the argsort + ``_seg_table`` of ponyexl3/mlx/exl3_moe.py:
+    79-98, 700-716). Returns int32 tensors (order, tok, sidx, table (n_blocks, 4))."""
+    _check_cuda(indices, "indices")
+    if indices.dtype != torch.int32 or indices.dim() != 2 or not indices.is_contiguous():
+        raise ValueError("indices must be a contiguous int32 (tokens, top_k) tensor")
+    if n_experts > MOE_SORT_MAX_EXPERTS:
+        raise ValueError(f"moe_sort handles at most {MOE_SORT_MAX_EXPERTS} experts")
+    tokens, top_k = indices.shape
+    n = tokens * top_k
+    dev = indices.device
+    out = torch.empty((3, n), dtype=torch.int32, device=dev)
+    table = torch.empty((n // block_rows + n_experts, 4), dtype=torch.int32, device=dev)
+    rc = _lib.load().exl3_moe_sort(_ptr(indices), n, top_k, int(n_experts), int(block_rows),
+                                   _ptr(out[0]), _ptr(out[1]), _ptr(out[2]), _ptr(table),
+                                   table.shape[0], _stream())
+    _lib.check(rc, "exl3_moe_sort")
+    return out[0], out[1], out[2], table
+
+
+def moe_glu_rows(g, u, sidx, gu_svh, dn_suh, activation: int = 0):
+    """Per sorted row: finish gate and up (output Hadamard, per-expert svh), GLU,
+    rotate for the down projection (``exl3_moe_glu_rows``). g, u: (N, H) fp16."""
+    _half(g, "g")
+    _half(u, "u")
+    _half(gu_svh, "gu_svh")
+    _half(dn_suh, "dn_suh")
+    _check_cuda(sidx, "sidx")
+    n, h = g.shape
+    n_experts = dn_suh.shape[0]
+    if (u.shape != g.shape or not g.is_contiguous() or not u.is_contiguous() or h % 128
+            or sidx.dtype != torch.int32 or sidx.numel() != n
+            or tuple(gu_svh.shape) != (n_experts, 2 * h) or tuple(dn_suh.shape) != (n_experts, h)
+            or not gu_svh.is_contiguous() or not dn_suh.is_contiguous()):
+        raise ValueError("moe_glu_rows: inconsistent shapes")
+    out = torch.empty_like(g)
+    rc = _lib.load().exl3_moe_glu_rows(_ptr(g), _ptr(u), n, h, _ptr(sidx), _ptr(gu_svh), _ptr(dn_suh),
+                                       n_experts, int(activation), _ptr(out), _stream())
+    _lib.check(rc, "exl3_moe_glu_rows")
+    return out
+
+
 def gemm_grouped(xh, trellis, k: int, cb: int, tn_base: int, group_tiles: int, n_groups: int,
                  table: torch.Tensor, block_rows: int):
     """Segmented prefill GEMM: rows of ``xh`` (N, in) are sorted into groups, group g

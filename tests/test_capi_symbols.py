@@ -63,6 +63,12 @@ def test_argument_errors_before_launch(lib):
     assert lib.exl3_pack_trellis(p, 1, 0, p, None) == _lib.EXL3_E_BAD_K
     assert lib.exl3_pack_trellis(p, 1, 4, None, None) == _lib.EXL3_E_NULL_POINTER
     assert lib.exl3_pack_trellis(p, 0, 4, p, None) == _lib.EXL3_OK
+    assert lib.exl3_moe_sort(p, 8, 2, 4, 64, p, p, p, p, 3, None) == _lib.EXL3_E_BAD_SHAPE  # table too short
+    assert lib.exl3_moe_sort(p, 8, 2, 2000, 64, p, p, p, p, 4000, None) == _lib.EXL3_E_UNSUPPORTED
+    assert lib.exl3_moe_sort(p, 8, 2, 4, 64, p, p, None, p, 8, None) == _lib.EXL3_E_NULL_POINTER
+    assert lib.exl3_moe_glu_rows(p, p, 4, 100, p, p, p, 2, 0, p, None) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_moe_glu_rows(p, p, 4, 128, p, p, p, 2, 5, p, None) == _lib.EXL3_E_UNSUPPORTED
+    assert lib.exl3_moe_glu_rows(p, p, 0, 128, p, p, p, 2, 0, p, None) == _lib.EXL3_OK
     assert lib.exl3_decode_full_eg(p, 1, 6, 4, 0, 4, p, None) == _lib.EXL3_E_BAD_SHAPE
     assert lib.exl3_decode_full_eg(p, 1, 6, 4, 0, 0, p, None) == _lib.EXL3_E_BAD_SHAPE
     assert lib.exl3_decode_full_eg(p, 1, 6, 0, 0, 3, p, None) == _lib.EXL3_E_BAD_K

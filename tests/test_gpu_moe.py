@@ -212,3 +212,58 @@ def test_moe_block_with_shared_expert(cuda, oracle):
     per_expert = _oracle_chain(oracle, gate, up, down, x.numpy(), inds.astype(np.int32), "silu")
     ref = (per_expert.astype(np.float32) * scores[..., None]).sum(axis=1)
     assert rel_l2(y, ref) <= 2 * TOL  # fp16 products and sum over three experts on top of the chain
+
+
+@pytest.mark.parametrize("tokens,top_k,E,block_rows", [(40, 2, 7, 64), (513, 8, 256, 64), (3000, 4, 1024, 64),
+                                                        (2100, 8, 16, 256), (1, 1, 1, 64)])
+def test_pair_sort_kernel_equals_stable_argsort(cuda, tokens, top_k, E, block_rows):
+    """Integer work, bit-exact: order / tok / sidx against torch's stable argsort, the
+    row-block table against the table built from device-side torch ops (same worst-case
+    length, same empty entries). Includes out-of-range ids (clamped), experts with no
+    pair and more pairs than one 1024-pair scatter round."""
+    from ponyexl3_amd import ops
+
+    rng = np.random.default_rng(tokens + E)
+    idx = rng.integers(0, E, size=(tokens, top_k)).astype(np.int32)
+    if E > 4:
+        idx[idx == 3] = 2  # expert 3 gets nothing
+        idx[0, 0] = E + 5  # clamps to E - 1
+        if tokens > 1:
+            idx[1, 0] = -4  # clamps to 0
+    it = torch.from_numpy(idx).to(cuda)
+    order, tok, sidx, table = ops.moe_sort(it, E, block_rows)
+    flat = it.reshape(-1).long().clamp(0, E - 1)
+    ref_order = torch.argsort(flat, stable=True)
+    assert torch.equal(order.long(), ref_order)
+    assert torch.equal(sidx.long(), flat[ref_order])
+    assert torch.equal(tok.long(), ref_order // top_k)
+    ref_table = ops.segment_table(flat[ref_order], E, block_rows)
+    assert tuple(table.shape) == tuple(ref_table.shape)
+    assert torch.equal(table, ref_table)
+    o2, t2, s2, tab2 = ops.moe_sort(it, E, block_rows)  # same answer every call
+    assert torch.equal(o2, order) and torch.equal(tab2, table)
+
+
+@pytest.mark.parametrize("act", [0, 1])
+def test_glu_rows_kernel_equals_separate_launches(cuda, act):
+    """Finish gate/up + GLU + down rotation in one launch against the per-row
+    Hadamard launches around torch's GLU (same casts: fp16 after every stage)."""
+    from ponyexl3_amd import ops
+
+    rng = np.random.default_rng(17 + act)
+    N, H, E = 300, 384, 9
+    g = torch.from_numpy((rng.standard_normal((N, H)) * 2).astype(np.float16)).to(cuda)
+    u = torch.from_numpy((rng.standard_normal((N, H)) * 2).astype(np.float16)).to(cuda)
+    sidx = torch.from_numpy(np.sort(rng.integers(0, E, size=N)).astype(np.int32)).to(cuda)
+    sgn = lambda *s: torch.from_numpy(np.where(rng.random(s) > 0.5, -1, 1).astype(np.float16)).to(cuda)
+    gu_svh, dn_suh = sgn(E, 2 * H), sgn(E, H)
+    got = ops.moe_glu_rows(g, u, sidx, gu_svh, dn_suh, act)
+    gf = ops.had128_rows(g, gu_svh[:, :H], True, scale_index=sidx).float()
+    uf = ops.had128_rows(u, gu_svh[:, H:], True, scale_index=sidx).float()
+    a = torch.nn.functional.gelu(gf, approximate="tanh") if act else torch.nn.functional.silu(gf)
+    ref = ops.had128_rows((a * uf).to(torch.float16), dn_suh, False, scale_index=sidx)
+    diff = (got.float() - ref.float()).abs().max()
+    # expf / tanhf of the kernel vs torch's: an fp16 ulp of h here and there
+    assert float(diff) <= 4e-3 * float(ref.float().abs().max())
+    with pytest.raises(ValueError):
+        ops.moe_glu_rows(g, u[:, :256], sidx, gu_svh, dn_suh, act)
