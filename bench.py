@@ -367,11 +367,12 @@ def _rows_x(n, rows, dev):
 
 
 def bench_batch_rows(dev, layer):
-    """The same layer step at 2, 4 and 8 rows (batched decode, speculative verify):
-    sum of the four launch durations on cold weights."""
+    """The same layer step at 2, 4, 8 and 16 rows (batched decode, speculative verify):
+    sum of the launch durations on cold weights (at 16 rows each linear is the input
+    rotation launch plus the one-launch kernel)."""
     res = {}
     total = sum(l.bytes for l in layer)
-    for rows in (2, 4, 8):
+    for rows in (2, 4, 8, 16):
         ms = sum(_launch_ms(lin, _rows_x(lin.n_in, rows, dev), K_BITS, dev) for lin in layer)
         res[f"rows_{rows}"] = {"us_per_step": round(ms * 1e3, 2), "GBps": round(total / ms / 1e6, 1)}
     return {"batch_rows": res}

@@ -49,6 +49,11 @@ const char *exl3_status_string(int status);
 /* Largest row count the small-batch kernel (exl3_gemv) accepts per call. */
 int exl3_gemv_max_rows(void);
 
+/* Largest row count exl3_linear_forward serves with its one-launch small-batch
+ * kernel when given counters (above exl3_gemv_max_rows() the input rotation runs
+ * as a launch of its own first). Beyond it the prefill GEMM takes over. */
+int exl3_linear_small_max_rows(void);
+
 /*
  * Trellis -> fp16 W_inner for a slice of tile columns.
  * Replaces decode_full_mlx (ponyexl3/mlx/gemv_metal.py:717-743) and the CPU

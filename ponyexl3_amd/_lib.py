@@ -32,6 +32,7 @@ PROTOTYPES = {
     "exl3_version": (_i, []),
     "exl3_status_string": (ctypes.c_char_p, [_i]),
     "exl3_gemv_max_rows": (_i, []),
+    "exl3_linear_small_max_rows": (_i, []),
     "exl3_decode_full": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _vp]),
     "exl3_moe_sort": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _vp]),
     "exl3_moe_glu_rows": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _vp, _vp]),

@@ -68,13 +68,16 @@ int launch_gemv_partials(const uint16_t* xh, int rows, int n_sub, const uint16_t
                          const int32_t* group_tile, int n_groups, float* partial, GemvPlan plan,
                          hipStream_t stream);
 
-// One-launch small-batch layer (rows <= kGemvMaxRows): counters[out_tiles/8] must
-// be zero on entry and are zero again on exit.
+// One-launch small-batch layer (rows <= kLinearSmallMaxRows): counters[out_tiles/8]
+// must be zero on entry and are zero again on exit. Up to kGemvMaxRows rows the
+// kernel rotates x itself (pre_rotated = false); above that x must be the output
+// of launch_had_pre, fp16 [rows][n_sub][in] (pre_rotated = true, suh not applied).
+constexpr int kLinearSmallMaxRows = 16;
 int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, int in_tiles,
                         int out_tiles, int K, int cb, const uint16_t* suh, int n_sub,
                         const int32_t* group_sub, const uint16_t* svh, const uint16_t* bias,
                         uint16_t* y, float* partial, int* counters, GemvPlan plan,
-                        hipStream_t stream);
+                        bool pre_rotated, hipStream_t stream);
 
 int launch_had_pre(const uint16_t* x, int rows, int n, const uint16_t* suh, int n_sub,
                    uint16_t* xh, hipStream_t stream);

@@ -10,6 +10,11 @@ namespace exl3 {
 
 constexpr float kHadScaleF = 0.088388347648318440550f;  // 1/sqrt(128)
 
+// Row stride (halfs) of a wave's staged activation block [MT][kXwLd]: 128 values
+// plus 16 bytes, so that the four batch rows a quad of lanes reads with one
+// ds_read_b128 start four LDS banks apart instead of in the same bank.
+constexpr int kXwLd = 136;
+
 template <int K>
 __device__ __forceinline__ void load_lane_words_nt(const uint32_t* __restrict__ p,
                                                    uint32_t (&own)[K]) {
@@ -38,7 +43,7 @@ __device__ __forceinline__ void wht128_lanes(float& a, float& b, int lane) {
 // of the 8 tile columns that start at `base` (already offset by lane*K dwords)
 // and accumulates acc[m][0..1] += x[m][rows of the tile] . W[:, column u / u+8].
 //
-// Activations enter through the wave's own LDS slot xw[MT][128], one 128-wide
+// Activations enter through the wave's own LDS slot xw[MT][kXwLd], one 128-wide
 // block (8 tile rows) at a time:
 //   ROTATE  xw = fp16(had128(x * suh) / sqrt(128))   (ponyexl3/ref/forward.py:32-34)
 //   else    xw = x                                   (x is already rotated)
@@ -50,7 +55,7 @@ __device__ __forceinline__ void stream_block_rows(const uint32_t* __restrict__ b
                                                   size_t row_words, int tk_begin, int tk_end,
                                                   const half_t* __restrict__ x, size_t x_stride,
                                                   int rows, const half_t* __restrict__ suh_row,
-                                                  half_t (*xw)[128], int lane,
+                                                  half_t (*xw)[kXwLd], int lane,
                                                   float (&acc)[MT][2]) {
     half2_t xraw[MT], sraw;
     auto fetch_block = [&](int blk) {
@@ -114,19 +119,20 @@ __device__ __forceinline__ void stream_block_rows(const uint32_t* __restrict__ b
         const LaneWords<K> lw = make_lane_words<K>(prev, words);
         half2_t wp[16];
         decode_lane<K, CB>(lw, wp);
+        // fresh-row groups outermost: consecutive MFMAs then write 2*NQ different
+        // accumulators, so none waits for the one just issued
 #pragma unroll
-        for (int q = 0; q < NQ; q++) {
-            const uint4_t x0 = xt.q[q][0], x1 = xt.q[q][1];
-            const uint2_t xa[4] = {uint2_t{x0.x, x0.y}, uint2_t{x0.z, x0.w}, uint2_t{x1.x, x1.y},
-                                   uint2_t{x1.z, x1.w}};
+        for (int j4 = 0; j4 < 4; j4++) {  // input rows 4*j4 .. 4*j4+3 of the tile
 #pragma unroll
-            for (int j4 = 0; j4 < 4; j4++) {  // input rows 4*j4 .. 4*j4+3 of the tile
+            for (int q = 0; q < NQ; q++) {
+                const uint4_t xv = xt.q[q][j4 >> 1];
+                const uint2_t xa = (j4 & 1) ? uint2_t{xv.z, xv.w} : uint2_t{xv.x, xv.y};
 #pragma unroll
                 for (int cs = 0; cs < 2; cs++) {
                     const uint2_t wb = {half2_to_bits(wp[8 * cs + 2 * j4]),
                                         half2_to_bits(wp[8 * cs + 2 * j4 + 1])};
                     accv[cs][q] = __builtin_amdgcn_mfma_f32_4x4x4f16(
-                        __builtin_bit_cast(half4_t, xa[j4]), __builtin_bit_cast(half4_t, wb),
+                        __builtin_bit_cast(half4_t, xa), __builtin_bit_cast(half4_t, wb),
                         accv[cs][q], 0, 0, 0);
                 }
             }

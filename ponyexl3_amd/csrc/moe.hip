@@ -222,7 +222,7 @@ __global__ __launch_bounds__(256) void moe_gateup_kernel(
     const int* __restrict__ indices, const half_t* __restrict__ gu_suh,
     const half_t* __restrict__ gu_svh, const half_t* __restrict__ dn_suh, half_t* xh_dn,
     float* part, int* counters, int top_k, int E, int D, int H, int activation) {
-    __shared__ __attribute__((aligned(16))) half_t xs[4][1][128];
+    __shared__ __attribute__((aligned(16))) half_t xs[4][1][kXwLd];
     __shared__ float red[4][128];
     __shared__ float up_val[128];
     __shared__ int last_flag;
@@ -289,7 +289,7 @@ __global__ __launch_bounds__(256) void moe_down_kernel(
     const uint32_t* __restrict__ dn_trellis, const half_t* __restrict__ xh_dn,
     const int* __restrict__ indices, const half_t* __restrict__ dn_svh, half_t* __restrict__ y,
     float* part, int* counters, int E, int D, int H) {
-    __shared__ __attribute__((aligned(16))) half_t xs[4][1][128];
+    __shared__ __attribute__((aligned(16))) half_t xs[4][1][kXwLd];
     __shared__ float red[4][128];
     __shared__ int last_flag;
     const int lane = threadIdx.x & 63;

@@ -276,6 +276,11 @@ def gemv_max_rows() -> int:
     return int(_lib.load().exl3_gemv_max_rows())
 
 
+def linear_small_max_rows() -> int:
+    """Rows up to which ``linear_forward(fused=True)`` uses the one-launch kernel."""
+    return int(_lib.load().exl3_linear_small_max_rows())
+
+
 def group_sub_from_tile_sub(tile_sub) -> torch.Tensor:
     """tile_sub (out_tiles,) -> per-128-column table; every run of 8 tiles must
     share one member (members have out_features % 128 == 0)."""
@@ -541,7 +546,7 @@ def linear_forward(x2d, trellis, k, cb, suh=None, svh=None, bias=None, group_sub
     """Whole-layer forward on (rows, in) fp16 (``exl3_linear_forward``).
     ``fused=False`` selects the three-launch chain for small batches.
     ``member_out`` (out_features of each sibling, in order) is needed for a
-    sibling-fused group above ``gemv_max_rows()`` rows: the prefill GEMM runs once
+    sibling-fused group above ``linear_small_max_rows()`` rows: the prefill GEMM runs once
     per member over its tile columns, each on its own rotated activations
     (``FusedEXL3Group.forward_all``, ponyexl3/mlx/exl3_fused.py:136-202)."""
     in_tiles, out_tiles = _trellis_dims(trellis, k)
@@ -572,7 +577,7 @@ def linear_forward(x2d, trellis, k, cb, suh=None, svh=None, bias=None, group_sub
     y = torch.empty((rows, n_out), dtype=torch.float16, device=x2d.device)
     if rows == 0:
         return y
-    if n_sub > 1 and rows > gemv_max_rows():
+    if n_sub > 1 and rows > (linear_small_max_rows() if fused else gemv_max_rows()):
         if member_out is None or len(member_out) != n_sub or sum(member_out) != n_out:
             raise ValueError("member_out must list the out_features of the stacked members")
         xh = had128_pre(x2d, suh)  # (rows, n_sub, in)
