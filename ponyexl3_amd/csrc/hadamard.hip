@@ -88,7 +88,8 @@ __device__ __forceinline__ void halfs_to_floats(uint4_t q, float (&v)[8]) {
 }
 
 // Wide forms: grid.x = number of output rows ((row, sub) pairs for the input side);
-// the four waves of a workgroup take consecutive 512-element chunks of the row.
+// the four waves of a workgroup take consecutive 512-element chunks of the row,
+// and grid.y workgroups share a row when there are too few rows to fill the chip.
 // All pointers 16-byte aligned, n a multiple of 128.
 __global__ __launch_bounds__(256) void had_pre_wide_kernel(const half_t* __restrict__ x,
                                                            const half_t* __restrict__ suh,
@@ -103,7 +104,7 @@ __global__ __launch_bounds__(256) void had_pre_wide_kernel(const half_t* __restr
         suh ? suh + (map.per_row ? map.scale_row(rs) * map.scale_ld : (rs % n_sub) * (size_t)n)
             : nullptr;
     half_t* orow = xh + map.out_row(rs) * (size_t)n;
-    for (int c = threadIdx.x * 8; c < n; c += 2048) {
+    for (int c = (blockIdx.y * 256 + threadIdx.x) * 8; c < n; c += 2048 * gridDim.y) {
         float v[8], sv[8];
         halfs_to_floats(*reinterpret_cast<const uint4_t*>(xr + c), v);
         if (sr) {
@@ -134,7 +135,7 @@ __global__ __launch_bounds__(256) void had_post_wide_kernel(const half_t* __rest
     if (svh && map.per_row) svh += map.scale_row(rs) * map.scale_ld;
     const half_t* yr = y + map.in_row(rs) * (size_t)n;
     half_t* orow = out + map.out_row(rs) * (size_t)n;
-    for (int c = threadIdx.x * 8; c < n; c += 2048) {
+    for (int c = (blockIdx.y * 256 + threadIdx.x) * 8; c < n; c += 2048 * gridDim.y) {
         float v[8], sv[8];
         halfs_to_floats(*reinterpret_cast<const uint4_t*>(yr + c), v);
         wht128_wide(v, lane);
@@ -261,6 +262,15 @@ __global__ __launch_bounds__(256) void had_post_kernel(const void* __restrict__ 
 constexpr int kWideMinRows = 16;
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// Workgroups per row of the wide kernels: about four workgroups per CU in total,
+// never more than the row has 2048-element chunks.
+static unsigned wide_row_parts(long long rows, int n) {
+    const long long chunks = (n + 2047) / 2048;
+    long long want = (1024 + rows - 1) / rows;
+    if (want > chunks) want = chunks;
+    return (unsigned)(want < 1 ? 1 : want);
+}
+
 int launch_had_pre(const uint16_t* x, int rows, int n, const uint16_t* suh, int n_sub,
                    uint16_t* xh, hipStream_t stream) {
     if (!x || !xh) return EXL3_E_NULL_POINTER;
@@ -272,7 +282,8 @@ int launch_had_pre(const uint16_t* x, int rows, int n, const uint16_t* suh, int 
     if (grid > 0x7FFFFFFFLL) return EXL3_E_BAD_SHAPE;
     if ((long long)rows * n_sub >= kWideMinRows && aligned16(x) && aligned16(xh) &&
         (!suh || aligned16(suh))) {
-        had_pre_wide_kernel<<<dim3((unsigned)(rows * n_sub)), dim3(256), 0, stream>>>(
+        had_pre_wide_kernel<<<dim3((unsigned)(rows * n_sub), wide_row_parts((long long)rows * n_sub, n)),
+                              dim3(256), 0, stream>>>(
             reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(suh),
             reinterpret_cast<half_t*>(xh), n, n_sub, RowMap{});
         return launch_status();
@@ -297,7 +308,7 @@ int launch_had_post(const void* y, int y_is_fp32, int n_sum, size_t sum_stride, 
     half_t* o = reinterpret_cast<half_t*>(out);
     if (!y_is_fp32 && rows >= kWideMinRows && aligned16(y) && aligned16(out) &&
         (!svh || aligned16(svh)) && (!bias || aligned16(bias))) {
-        had_post_wide_kernel<<<dim3((unsigned)rows), dim3(256), 0, stream>>>(
+        had_post_wide_kernel<<<dim3((unsigned)rows, wide_row_parts(rows, n)), dim3(256), 0, stream>>>(
             reinterpret_cast<const half_t*>(y), s, b, o, n, RowMap{});
         return launch_status();
     }
@@ -320,11 +331,11 @@ int launch_had_rows(const uint16_t* x, int rows, int n, const int32_t* in_index,
     if (rows == 0) return EXL3_OK;
     const RowMap map{1, in_index, scale_index, out_index, scale_ld};
     if (post)
-        had_post_wide_kernel<<<dim3((unsigned)rows), dim3(256), 0, stream>>>(
+        had_post_wide_kernel<<<dim3((unsigned)rows, wide_row_parts(rows, n)), dim3(256), 0, stream>>>(
             reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(scale), nullptr,
             reinterpret_cast<half_t*>(out), n, map);
     else
-        had_pre_wide_kernel<<<dim3((unsigned)rows), dim3(256), 0, stream>>>(
+        had_pre_wide_kernel<<<dim3((unsigned)rows, wide_row_parts(rows, n)), dim3(256), 0, stream>>>(
             reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(scale),
             reinterpret_cast<half_t*>(out), n, 1, map);
     return launch_status();
