@@ -116,10 +116,13 @@ EXL3_EXPORT int exl3_linear_forward(const uint16_t* x, int rows, const uint16_t*
     }
     uint16_t* ytmp = reinterpret_cast<uint16_t*>(second);
     if (n_sub == 1) {
+        const GemmPost post{svh, bias, y, (size_t)out_features};
+        bool post_done = false;
         if (int rc = launch_gemm(xh, rows, (size_t)in_features, trellis, in_tiles, out_tiles, K, cb,
                                  0, out_tiles, ytmp, (size_t)out_features,
-                                 second + ws.second_bytes, ws.gemm_bytes, s))
+                                 second + ws.second_bytes, ws.gemm_bytes, s, &post, &post_done))
             return rc;
+        if (post_done) return EXL3_OK;  // few rows: the fix-up pass applied the output transform
     } else {
         return EXL3_E_UNSUPPORTED;  // fused groups run their members one by one on the host side
     }

@@ -98,10 +98,24 @@ struct GemmPlan {
 GemmPlan plan_gemm(int rows, int in_tiles, int tn_count, bool allow_split);
 size_t gemm_workspace_bytes(int rows, int in_tiles, int tn_count);
 
-// workspace may be NULL (or too small): then no tile is split.
+// Output transform the GEMM may fold into its fix-up pass: when every tile of the
+// launch is split along the reduction dimension (few rows), the kernel that adds
+// the partial tiles also applies the output Hadamard, svh and bias and writes
+// `out` [rows][ldo] directly (tn_offset must be 0 and tn_count the whole width).
+struct GemmPost {
+    const uint16_t* svh;   // fp16 [16*tn_count] or NULL
+    const uint16_t* bias;  // fp16 [16*tn_count] or NULL
+    uint16_t* out;
+    size_t ldo;
+};
+
+// workspace may be NULL (or too small): then no tile is split. If `post` is given
+// and could be applied, *post_done is set and y_out is left untouched; otherwise
+// y_out holds the plain product and the caller runs the output transform.
 int launch_gemm(const uint16_t* xh, int rows, size_t ldx, const uint16_t* trellis, int in_tiles,
                 int out_tiles, int K, int cb, int tn_offset, int tn_count, uint16_t* y_out,
-                size_t ldy, void* workspace, size_t workspace_bytes, hipStream_t stream);
+                size_t ldy, void* workspace, size_t workspace_bytes, hipStream_t stream,
+                const GemmPost* post = nullptr, bool* post_done = nullptr);
 
 int launch_gemm_grouped(const uint16_t* xh, int n_rows, size_t ldx, const uint16_t* trellis,
                         int in_tiles, int out_tiles, int K, int cb, int tn_base, int group_tiles,

@@ -360,6 +360,79 @@ __global__ __launch_bounds__(256) void gemm_fixup_kernel(const float* __restrict
     }
 }
 
+// The fix-up with the output transform folded in (every tile of the launch split):
+// a wave finishes one row of the tile's 256 columns, i.e. two Hadamard blocks, one
+// per half-wave, four values per lane. Same steps as the separate kernels: sum in
+// range order, one cast to fp16, fp32 butterflies in ascending stride, scale, svh,
+// cast, bias.
+template <int MI>
+__global__ __launch_bounds__(256) void gemm_fixup_post_kernel(
+    const float* __restrict__ partial, int rows, int tn_count, int n_row_blocks, int split,
+    const half_t* __restrict__ svh, const half_t* __restrict__ bias, half_t* __restrict__ out,
+    size_t ldo) {
+    constexpr int BM = 32 * MI;
+    constexpr float kScale = 0.088388347648318440550f;  // 1/sqrt(128)
+    const int tile = blockIdx.x;
+    const int g = tile / n_row_blocks;
+    const int m0 = (tile % n_row_blocks) * BM;
+    const int lane = threadIdx.x & 63;
+    const int c4 = lane * 4;
+    const int col = g * kGemmBN + c4;
+    const bool col_ok = col < tn_count * 16;  // false in the upper half of a half-width last block
+    const float* p0 = partial + (size_t)blockIdx.x * split * (BM * kGemmBN);
+#pragma unroll
+    for (int it = 0; it < 2; it++) {
+        const int rl = blockIdx.y * 8 + it * 4 + (threadIdx.x >> 6);
+        if (m0 + rl >= rows) return;  // whole wave
+        float4_t s = {0.f, 0.f, 0.f, 0.f};
+        if (col_ok) {
+            const float* p = p0 + rl * kGemmBN + c4;
+            s = *reinterpret_cast<const float4_t*>(p);
+            for (int sp = 1; sp < split; sp++)
+                s = s + *reinterpret_cast<const float4_t*>(p + (size_t)sp * (BM * kGemmBN));
+        }
+        float v[4] = {(float)(half_t)s.x, (float)(half_t)s.y, (float)(half_t)s.z,
+                      (float)(half_t)s.w};
+#pragma unroll
+        for (int h = 1; h < 4; h <<= 1) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if ((j & h) == 0) {
+                    const float lo = v[j], hi = v[j + h];
+                    v[j] = __fadd_rn(lo, hi);
+                    v[j + h] = __fsub_rn(lo, hi);
+                }
+            }
+        }
+#pragma unroll
+        for (int bit = 0; bit < 5; bit++) {
+            const int mask = 1 << bit;
+            const bool upper = (lane & mask) != 0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float q = __shfl_xor(v[j], mask, kWave);
+                v[j] = upper ? __fsub_rn(q, v[j]) : __fadd_rn(v[j], q);
+            }
+        }
+        if (col_ok) {
+            half_t o[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float a = __fmul_rn(v[j], kScale);
+                if (svh) a = __fmul_rn(a, (float)svh[col + j]);
+                o[j] = (half_t)a;
+                if (bias) o[j] = o[j] + bias[col + j];
+            }
+            half4_t ov;
+            ov.x = o[0];
+            ov.y = o[1];
+            ov.z = o[2];
+            ov.w = o[3];
+            *reinterpret_cast<half4_t*>(out + (size_t)(m0 + rl) * ldo + col) = ov;
+        }
+    }
+}
+
 static int gemm_slots() {
     // one workgroup per CU; the count only shapes the schedule, never the result of a tile
     static const int cus = [] {
@@ -390,7 +463,7 @@ GemmPlan plan_gemm(int rows, int in_tiles, int tn_count, bool allow_split) {
         // Cost of the last round in tile times: its workgroups run in
         // ceil(rem*s/slots) waves of 1/s tile each, and every range also writes (and
         // the fix-up reads) one fp32 tile, about the time of 8 steps.
-        const int max_split = env_int("EXL3_GEMM_MAX_SPLIT", 8, 1, 64);
+        const int max_split = env_int("EXL3_GEMM_MAX_SPLIT", 16, 1, 64);
         const double partial_cost = 8.0 / ksteps;
         double best = 1.0;
         for (int s = 2; s <= max_split && ksteps / s >= 4; s++) {
@@ -419,7 +492,7 @@ template <int K, int CB, int MI>
 static int launch_gemm_mi(const GemmPlan& p, const uint16_t* xh, int rows, size_t ldx,
                           const uint16_t* trellis, int in_tiles, int out_tiles, int tn_offset,
                           int tn_count, uint16_t* y_out, size_t ldy, float* partial,
-                          hipStream_t stream) {
+                          hipStream_t stream, const GemmPost* post) {
     constexpr size_t lds = (2 * (size_t)(32 * MI) * 64 + 2 * (size_t)kGemmStageB) * sizeof(half_t);
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_kernel<K, CB, MI>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -430,6 +503,13 @@ static int launch_gemm_mi(const GemmPlan& p, const uint16_t* xh, int rows, size_
         reinterpret_cast<half_t*>(y_out), partial, rows, ldx, ldy, in_tiles, out_tiles, tn_offset,
         tn_count, p.n_row_blocks, p.full_tiles, p.split, p.ksteps_per_split, nullptr, 0);
     if (int rc = launch_status()) return rc;
+    if (post) {  // only passed when every tile is split
+        gemm_fixup_post_kernel<MI><<<dim3((unsigned)p.split_tiles, 4 * MI), dim3(256), 0, stream>>>(
+            partial, rows, tn_count, p.n_row_blocks, p.split,
+            reinterpret_cast<const half_t*>(post->svh), reinterpret_cast<const half_t*>(post->bias),
+            reinterpret_cast<half_t*>(post->out), post->ldo);
+        return launch_status();
+    }
     if (p.split_tiles > 0) {
         gemm_fixup_kernel<MI><<<dim3((unsigned)p.split_tiles, 4 * MI), dim3(256), 0, stream>>>(
             partial, reinterpret_cast<half_t*>(y_out), rows, ldy, tn_count, p.n_row_blocks,
@@ -441,7 +521,9 @@ static int launch_gemm_mi(const GemmPlan& p, const uint16_t* xh, int rows, size_
 
 int launch_gemm(const uint16_t* xh, int rows, size_t ldx, const uint16_t* trellis, int in_tiles,
                 int out_tiles, int K, int cb, int tn_offset, int tn_count, uint16_t* y_out,
-                size_t ldy, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+                size_t ldy, void* workspace, size_t workspace_bytes, hipStream_t stream,
+                const GemmPost* post, bool* post_done) {
+    if (post_done) *post_done = false;
     if (int rc = check_k_cb(K, cb)) return rc;
     if (!xh || !trellis || !y_out) return EXL3_E_NULL_POINTER;
     if (rows < 1 || in_tiles < 4 || in_tiles % 4 || tn_offset < 0 || tn_count < 8 ||
@@ -458,19 +540,26 @@ int launch_gemm(const uint16_t* xh, int rows, size_t ldx, const uint16_t* trelli
     if ((long long)p.full_tiles + (long long)p.split_tiles * p.split > 0x7fffffffLL)
         return EXL3_E_BAD_SHAPE;
     float* partial = reinterpret_cast<float*>(workspace);
-    return dispatch_k_cb(K, cb, [&](auto k, auto c) {
+    // the output transform rides on the fix-up when there is nothing but split tiles
+    const bool fold = post && post->out && post_done && p.split > 1 && p.full_tiles == 0 &&
+                      tn_offset == 0 && post->ldo >= (size_t)tn_count * 16 && post->ldo % 4 == 0 &&
+                      !(reinterpret_cast<uintptr_t>(post->out) & 7);
+    const GemmPost* fp = fold ? post : nullptr;
+    const int rc = dispatch_k_cb(K, cb, [&](auto k, auto c) {
         if (p.mi == 2)
             return launch_gemm_mi<k.value, c.value, 2>(p, xh, rows, ldx, trellis, in_tiles,
                                                        out_tiles, tn_offset, tn_count, y_out, ldy,
-                                                       partial, stream);
+                                                       partial, stream, fp);
         if (p.mi == 4)
             return launch_gemm_mi<k.value, c.value, 4>(p, xh, rows, ldx, trellis, in_tiles,
                                                        out_tiles, tn_offset, tn_count, y_out, ldy,
-                                                       partial, stream);
+                                                       partial, stream, fp);
         return launch_gemm_mi<k.value, c.value, 8>(p, xh, rows, ldx, trellis, in_tiles, out_tiles,
                                                    tn_offset, tn_count, y_out, ldy, partial,
-                                                   stream);
+                                                   stream, fp);
     });
+    if (rc == EXL3_OK && fold) *post_done = true;
+    return rc;
 }
 
 template <int K, int CB, int MI>

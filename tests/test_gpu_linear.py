@@ -220,3 +220,26 @@ def test_one_launch_layer_equals_three_launch_chain(cuda, rows, k, n_in, n_out):
         diff = float((a.float() - b.float()).abs().max())
         assert diff <= 2e-3 * float(b.float().abs().max()), f"rep {rep}: {diff}"
     assert int(ops.sync_counters(cuda, 1).abs().sum()) == 0
+
+
+@pytest.mark.parametrize("rows", [17, 33, 64, 100, 130])
+@pytest.mark.parametrize("k,n_in,n_out", [(4, 2176, 640), (3, 4096, 384), (5, 1024, 1280)])
+def test_prefill_rows_with_every_tile_split(cuda, oracle, rows, k, n_in, n_out):
+    """Few rows and few column blocks: every GEMM tile is split along the reduction
+    dimension and the pass that adds the partial tiles also applies the output
+    Hadamard, svh and bias. 640 and 384 columns end in a half-width block. Checked
+    against the oracle and against the separate GEMM + output-transform launches."""
+    from ponyexl3_amd import make_exl3_layer, ops
+
+    layer = make_exl3_layer(k=k, in_features=n_in, out_features=n_out, seed=3 * k + rows, mcg=True, bias=True)
+    cb = int(layer.codebook_mode)
+    tr = ops.as_trellis_tensor(layer.trellis, cuda)
+    suh, svh = torch.from_numpy(layer.suh).to(cuda), torch.from_numpy(layer.svh).to(cuda)
+    bias = torch.from_numpy(layer.bias).to(cuda)
+    rng = np.random.default_rng(rows + n_in)
+    x, xt = _x(rng, (rows, n_in), cuda)
+    print(f"split prefill rows={rows} k={k} {n_in}->{n_out}", flush=True)
+    y = ops.linear_forward(xt, tr, k, cb, suh, svh, bias, fused=False)
+    assert rel_l2(y.cpu().numpy(), _oracle_forward(oracle, layer, x)) <= TOL
+    parts = ops.had128_post(ops.inner_gemm(ops.had128_pre(xt, suh), tr, k, cb), svh, bias)
+    assert torch.equal(y, parts)
