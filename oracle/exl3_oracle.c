@@ -37,12 +37,13 @@
  *                          chain as a whole is "parity unpinned" beyond that.
  *   exl3o_quantize_tile_exact
  *                          exact Viterbi over the bitshift trellis
- *                          (convert/reference_search.py). Pinned by what the
- *                          mathematics fixes: brute force over every closed path
- *                          of a short trellis, recovery of exactly representable
- *                          tiles, the tail-biting closure, pack -> unpack round
- *                          trip of its states (the reference's own assertions,
- *                          tests/test_convert_metal.py:25-86).
+ *                          (convert/reference_search.py). Pinned: states and
+ *                          decoded values written by the reference's
+ *                          quantize_tile_reference for six (K, codebook) cases
+ *                          (tests/golden/search_exact.npz, bit-exact, closing
+ *                          passes and tie-breaking included); brute force over
+ *                          every path of a short trellis; recovery of exactly
+ *                          representable tiles; chain validity of the states.
  *   exl3o_quantize_tiles_search
  *                          the production search kernel's arithmetic
  *                          (convert/metal_search.py:63-196: compressed states,

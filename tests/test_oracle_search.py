@@ -136,3 +136,17 @@ def test_search_argument_errors(oracle):
     q, idx = oracle.quantize_tiles_search(np.zeros((3, 256), dtype=np.float32), 4, DEFAULT)
     assert q.shape == (3, 256) and idx.shape == (3, 256)
     assert (idx[0] == idx[1]).all() and (idx[1] == idx[2]).all()
+
+
+@pytest.mark.parametrize("k,cb", [(2, MCG), (3, MCG), (4, DEFAULT), (4, MCG), (4, MUL1), (5, MCG)])
+def test_exact_search_equals_reference_vectors(oracle, k, cb):
+    """States and decoded values written by the reference's quantize_tile_reference
+    (tests/golden/make_golden_search.py): same path bit for bit, including the
+    closing passes and the tie-breaking."""
+    from conftest import golden
+
+    g = golden("search_exact.npz")
+    tag = f"k{k}_cb{cb}"
+    states, decoded = oracle.quantize_tile_exact(g[tag + "_tile"], k, cb)
+    np.testing.assert_array_equal(states, g[tag + "_states"])
+    np.testing.assert_array_equal(decoded.view(np.uint32), g[tag + "_decoded"].view(np.uint32))
