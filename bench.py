@@ -146,6 +146,9 @@ def main():
     ap.add_argument("--unfused-qkv", action="store_true", help="run q, k, v as three launches")
     ap.add_argument("--sweep", action="store_true",
                     help="also time config 5: the layer at K in {2,3,5,6,8}, 3INST and MCG, 1/4/8 rows")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one 64 MiB device-to-device copy (for counter runs: FETCH_SIZE / "
+                         "WRITE_SIZE of a transfer of known size)")
     args = ap.parse_args()
     global LAYER
     if args.unfused_qkv:
@@ -163,6 +166,14 @@ def main():
     _lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.copy_calibration:
+        src = torch.zeros(64 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     n_layers = max(1, args.layers)
     layers = [
