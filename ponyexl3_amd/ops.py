@@ -18,6 +18,9 @@ import torch
 from . import _lib
 
 _workspaces: dict = {}
+# Buffers that were replaced by larger ones stay allocated: a HIP graph captured
+# earlier still replays launches that point into them.
+_retired: list = []
 
 
 def _check_cuda(t: torch.Tensor, name: str) -> None:
@@ -44,6 +47,8 @@ def workspace(device, nbytes: int) -> torch.Tensor:
     key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
+        if buf is not None:
+            _retired.append(buf)
         buf = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = buf
     return buf
@@ -60,6 +65,8 @@ def gemm_workspace(device, nbytes: int):
     key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
     buf = _gemm_workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
+        if buf is not None:
+            _retired.append(buf)
         buf = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
         _gemm_workspaces[key] = buf
     return buf
@@ -74,6 +81,8 @@ def sync_counters(device, n: int) -> torch.Tensor:
     key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
     buf = _counters.get(key)
     if buf is None or buf.numel() < n:
+        if buf is not None:
+            _retired.append(buf)
         buf = torch.zeros(max(int(n), 4096), dtype=torch.int32, device=device)
         _counters[key] = buf
     return buf
