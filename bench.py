@@ -88,6 +88,9 @@ class DeviceLinear:
         if members > 1:
             gs = np.repeat(np.arange(members, dtype=np.int32), [o // 128 for o in outs])
             self.group_sub = torch.from_numpy(gs).to(device)
+        # member of every 256-column block (one-launch prefill GEMM of a sibling group)
+        self.block_sub = (self.group_sub[::2].contiguous()
+                          if members > 1 and all(o % 256 == 0 for o in outs) else None)
         self.bytes = weight_bytes(n_in, outs)
         self.outs = list(outs)
 
@@ -95,7 +98,8 @@ class DeviceLinear:
         from ponyexl3_amd import ops
 
         return ops.linear_forward(x, self.trellis, K_BITS, CB, self.suh, self.svh, None, self.group_sub,
-                                  member_out=self.outs if self.members > 1 else None)
+                                  member_out=self.outs if self.members > 1 else None,
+                                  block_sub=self.block_sub)
 
 
 def cpu_baseline(budget_s=12.0):

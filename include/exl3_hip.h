@@ -271,6 +271,24 @@ int exl3_moe_forward(const uint16_t *x, int tokens, const int32_t *indices, int 
 size_t exl3_moe_workspace_bytes(int tokens, int top_k, int D, int H);
 
 /*
+ * Prefill of one layer on activations that exl3_had128_pre already rotated:
+ * the MFMA trellis GEMM and the output transform (Hadamard-128, svh, bias), for a
+ * plain layer (n_sub = 1) or a sibling-fused one whose members all have
+ * out_features % 256 == 0. What FusedEXL3Group.forward_all does above the
+ * small-batch row counts (ponyexl3/mlx/exl3_fused.py:136-202) in one GEMM launch.
+ *   xh        fp16 [rows][n_sub][16*in_tiles]
+ *   block_sub i32 [out_tiles/16 rounded up] member index of every 256-column block
+ *             (required when n_sub > 1)
+ *   y         fp16 [rows][16*out_tiles]
+ *   workspace exl3_linear_prefill_workspace_bytes(rows, in, out) bytes
+ */
+size_t exl3_linear_prefill_workspace_bytes(int rows, int in_features, int out_features);
+int exl3_linear_prefill(const uint16_t *xh, int rows, int n_sub, const uint16_t *trellis,
+                        int in_tiles, int out_tiles, int K, int cb, const int32_t *block_sub,
+                        const uint16_t *svh, const uint16_t *bias, uint16_t *y, void *workspace,
+                        size_t workspace_bytes, void *stream);
+
+/*
  * MoE prefill glue, one launch each.
  * exl3_moe_sort: stable counting sort of the (token, slot) pairs by expert plus the
  * row-block table exl3_gemm_grouped takes. Replaces the argsort / segment-table

@@ -34,6 +34,8 @@ PROTOTYPES = {
     "exl3_gemv_max_rows": (_i, []),
     "exl3_linear_small_max_rows": (_i, []),
     "exl3_decode_full": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _vp]),
+    "exl3_linear_prefill_workspace_bytes": (_sz, [_i, _i, _i]),
+    "exl3_linear_prefill": (_i, [_vp, _i, _i, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "exl3_moe_sort": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _vp]),
     "exl3_moe_glu_rows": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "exl3_quantize_slot_bytes": (_sz, [_i]),

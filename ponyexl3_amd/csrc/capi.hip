@@ -128,3 +128,42 @@ EXL3_EXPORT int exl3_linear_forward(const uint16_t* x, int rows, const uint16_t*
     }
     return launch_had_post(ytmp, 0, 1, 0, rows, out_features, svh, bias, y, s);
 }
+
+// Prefill of a layer whose activations are already rotated: MFMA GEMM over
+// xh [rows][n_sub][in] (block_sub picks the rotation of every 256-column block when
+// n_sub > 1), then the output transform, folded into the GEMM's fix-up pass where
+// every tile is split.
+EXL3_EXPORT size_t exl3_linear_prefill_workspace_bytes(int rows, int in_features, int out_features) {
+    if (rows < 1 || in_features < 64 || out_features < 128) return 0;
+    using namespace exl3;
+    return align_up((size_t)rows * out_features * 2, 256) +
+           align_up(gemm_workspace_bytes(rows, in_features / 16, out_features / 16), 256);
+}
+
+EXL3_EXPORT int exl3_linear_prefill(const uint16_t* xh, int rows, int n_sub, const uint16_t* trellis,
+                                    int in_tiles, int out_tiles, int K, int cb,
+                                    const int32_t* block_sub, const uint16_t* svh,
+                                    const uint16_t* bias, uint16_t* y, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+    using namespace exl3;
+    if (int rc = check_k_cb(K, cb)) return rc;
+    if (!xh || !trellis || !y || !workspace) return EXL3_E_NULL_POINTER;
+    if (rows < 1 || in_tiles < 8 || out_tiles < 8 || in_tiles % 8 || out_tiles % 8 || n_sub < 1)
+        return EXL3_E_BAD_SHAPE;
+    if (n_sub > 1 && !block_sub) return EXL3_E_BAD_INDEX;
+    const int in_features = in_tiles * 16, out_features = out_tiles * 16;
+    const size_t y_bytes = align_up((size_t)rows * out_features * 2, 256);
+    const size_t g_bytes = align_up(gemm_workspace_bytes(rows, in_tiles, out_tiles), 256);
+    if (workspace_bytes < y_bytes + g_bytes) return EXL3_E_WORKSPACE;
+    hipStream_t s = as_stream(stream);
+    uint16_t* ytmp = reinterpret_cast<uint16_t*>(workspace);
+    const GemmPost post{svh, bias, y, (size_t)out_features};
+    bool post_done = false;
+    if (int rc = launch_gemm(xh, rows, (size_t)n_sub * in_features, trellis, in_tiles, out_tiles, K,
+                             cb, 0, out_tiles, ytmp, (size_t)out_features,
+                             reinterpret_cast<char*>(workspace) + y_bytes, g_bytes, s, &post,
+                             &post_done, n_sub > 1 ? block_sub : nullptr, (size_t)in_features))
+        return rc;
+    if (post_done) return EXL3_OK;
+    return launch_had_post(ytmp, 0, 1, 0, rows, out_features, svh, bias, y, s);
+}

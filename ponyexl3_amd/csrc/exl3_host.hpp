@@ -115,7 +115,11 @@ struct GemmPost {
 int launch_gemm(const uint16_t* xh, int rows, size_t ldx, const uint16_t* trellis, int in_tiles,
                 int out_tiles, int K, int cb, int tn_offset, int tn_count, uint16_t* y_out,
                 size_t ldy, void* workspace, size_t workspace_bytes, hipStream_t stream,
-                const GemmPost* post = nullptr, bool* post_done = nullptr);
+                const GemmPost* post = nullptr, bool* post_done = nullptr,
+                const int32_t* block_sub = nullptr, size_t sub_stride = 0);
+// block_sub (device, one entry per 256-column block of the slice, or NULL): the
+// block multiplies xh + block_sub[g] * sub_stride instead of xh (stacked rotations
+// of a sibling-fused layer).
 
 int launch_gemm_grouped(const uint16_t* xh, int n_rows, size_t ldx, const uint16_t* trellis,
                         int in_tiles, int out_tiles, int K, int cb, int tn_base, int group_tiles,

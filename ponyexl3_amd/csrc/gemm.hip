@@ -75,7 +75,8 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
     const uint32_t* __restrict__ trellis, const half_t* __restrict__ xh, half_t* __restrict__ y,
     float* __restrict__ partial, int rows_arg, size_t ldx, size_t ldy, int in_tiles, int out_tiles,
     int tn_offset_arg, int tn_count_arg, int n_row_blocks, int full_tiles, int split,
-    int ksteps_per_split, const int4* __restrict__ group_tab, int group_tiles) {
+    int ksteps_per_split, const int4* __restrict__ group_tab, int group_tiles,
+    const int* __restrict__ block_sub, size_t sub_stride) {
     extern __shared__ __attribute__((aligned(16))) half_t smem[];
     constexpr int BM = 32 * MI;
     constexpr int STAGE_A = BM * 64, STAGE_B = kGemmStageB;
@@ -111,6 +112,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
         rows = rows_arg;
         tn_offset = tn_offset_arg;
         tn_count = tn_count_arg;
+        // sibling-fused layers: every 256-column block multiplies the activations that
+        // were rotated with its own member's suh, xh[row][block_sub[g]][:]
+        if (block_sub) xh += (size_t)block_sub[g] * sub_stride;
     }
     const int k_begin = work.k_begin, k_last = work.k_end - 1;
     const int nsteps = work.k_end - work.k_begin;
@@ -492,7 +496,8 @@ template <int K, int CB, int MI>
 static int launch_gemm_mi(const GemmPlan& p, const uint16_t* xh, int rows, size_t ldx,
                           const uint16_t* trellis, int in_tiles, int out_tiles, int tn_offset,
                           int tn_count, uint16_t* y_out, size_t ldy, float* partial,
-                          hipStream_t stream, const GemmPost* post) {
+                          hipStream_t stream, const GemmPost* post, const int32_t* block_sub,
+                          size_t sub_stride) {
     constexpr size_t lds = (2 * (size_t)(32 * MI) * 64 + 2 * (size_t)kGemmStageB) * sizeof(half_t);
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_kernel<K, CB, MI>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -501,7 +506,8 @@ static int launch_gemm_mi(const GemmPlan& p, const uint16_t* xh, int rows, size_
     gemm_kernel<K, CB, MI><<<dim3(units), dim3(kGemmThreads), lds, stream>>>(
         reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<const half_t*>(xh),
         reinterpret_cast<half_t*>(y_out), partial, rows, ldx, ldy, in_tiles, out_tiles, tn_offset,
-        tn_count, p.n_row_blocks, p.full_tiles, p.split, p.ksteps_per_split, nullptr, 0);
+        tn_count, p.n_row_blocks, p.full_tiles, p.split, p.ksteps_per_split, nullptr, 0, block_sub,
+        sub_stride);
     if (int rc = launch_status()) return rc;
     if (post) {  // only passed when every tile is split
         gemm_fixup_post_kernel<MI><<<dim3((unsigned)p.split_tiles, 4 * MI), dim3(256), 0, stream>>>(
@@ -522,7 +528,8 @@ static int launch_gemm_mi(const GemmPlan& p, const uint16_t* xh, int rows, size_
 int launch_gemm(const uint16_t* xh, int rows, size_t ldx, const uint16_t* trellis, int in_tiles,
                 int out_tiles, int K, int cb, int tn_offset, int tn_count, uint16_t* y_out,
                 size_t ldy, void* workspace, size_t workspace_bytes, hipStream_t stream,
-                const GemmPost* post, bool* post_done) {
+                const GemmPost* post, bool* post_done, const int32_t* block_sub,
+                size_t sub_stride) {
     if (post_done) *post_done = false;
     if (int rc = check_k_cb(K, cb)) return rc;
     if (!xh || !trellis || !y_out) return EXL3_E_NULL_POINTER;
@@ -549,14 +556,14 @@ int launch_gemm(const uint16_t* xh, int rows, size_t ldx, const uint16_t* trelli
         if (p.mi == 2)
             return launch_gemm_mi<k.value, c.value, 2>(p, xh, rows, ldx, trellis, in_tiles,
                                                        out_tiles, tn_offset, tn_count, y_out, ldy,
-                                                       partial, stream, fp);
+                                                       partial, stream, fp, block_sub, sub_stride);
         if (p.mi == 4)
             return launch_gemm_mi<k.value, c.value, 4>(p, xh, rows, ldx, trellis, in_tiles,
                                                        out_tiles, tn_offset, tn_count, y_out, ldy,
-                                                       partial, stream, fp);
+                                                       partial, stream, fp, block_sub, sub_stride);
         return launch_gemm_mi<k.value, c.value, 8>(p, xh, rows, ldx, trellis, in_tiles, out_tiles,
                                                    tn_offset, tn_count, y_out, ldy, partial,
-                                                   stream, fp);
+                                                   stream, fp, block_sub, sub_stride);
     });
     if (rc == EXL3_OK && fold) *post_done = true;
     return rc;
@@ -577,7 +584,8 @@ static int launch_gemm_grouped_mi(const uint16_t* xh, int n_rows, size_t ldx,
     gemm_kernel<K, CB, MI><<<dim3((unsigned)units), dim3(kGemmThreads), lds, stream>>>(
         reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<const half_t*>(xh),
         reinterpret_cast<half_t*>(y_out), nullptr, n_rows, ldx, ldy, in_tiles, out_tiles, tn_base,
-        group_tiles, 1, 0, 1, in_tiles / 4, reinterpret_cast<const int4*>(group_tab), group_tiles);
+        group_tiles, 1, 0, 1, in_tiles / 4, reinterpret_cast<const int4*>(group_tab), group_tiles,
+        nullptr, 0);
     return launch_status();
 }
 

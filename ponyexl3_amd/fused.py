@@ -58,6 +58,9 @@ class FusedEXL3Group(torch.nn.Module):
         )
         self._tile_sub = tile_sub
         self._group_sub = ops.group_sub_from_tile_sub(tile_sub).to(device)
+        # member of every 256-column block, for the one-launch prefill GEMM
+        self._block_sub = (self._group_sub[::2].contiguous()
+                           if all(n % 256 == 0 for n in self._out_features) else None)
         self._cache_x = None
         self._cache_out = None
 
@@ -69,7 +72,7 @@ class FusedEXL3Group(torch.nn.Module):
         x2d = x.reshape(-1, self.in_features).to(torch.float16).contiguous()
         y = ops.linear_forward(
             x2d, self._trellis, self._k, self._cb, self._suh_stack, self._svh_cat, None,
-            self._group_sub, member_out=self._out_features,
+            self._group_sub, member_out=self._out_features, block_sub=self._block_sub,
         )
         outs = torch.split(y, self._out_features, dim=-1)
         return tuple(o.reshape(lead + (n,)) for o, n in zip(outs, self._out_features))

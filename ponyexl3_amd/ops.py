@@ -551,13 +551,15 @@ def gemm_grouped(xh, trellis, k: int, cb: int, tn_base: int, group_tiles: int, n
 
 
 def linear_forward(x2d, trellis, k, cb, suh=None, svh=None, bias=None, group_sub=None,
-                   fused: bool = True, member_out=None):
+                   fused: bool = True, member_out=None, block_sub=None):
     """Whole-layer forward on (rows, in) fp16 (``exl3_linear_forward``).
     ``fused=False`` selects the three-launch chain for small batches.
     ``member_out`` (out_features of each sibling, in order) is needed for a
     sibling-fused group above ``linear_small_max_rows()`` rows: the prefill GEMM runs once
     per member over its tile columns, each on its own rotated activations
-    (``FusedEXL3Group.forward_all``, ponyexl3/mlx/exl3_fused.py:136-202)."""
+    (``FusedEXL3Group.forward_all``, ponyexl3/mlx/exl3_fused.py:136-202), or once
+    over all members when each has ``out_features % 256 == 0`` (``block_sub``: the
+    member index of every 256-column block, derived from ``group_sub`` if absent)."""
     in_tiles, out_tiles = _trellis_dims(trellis, k)
     _half(x2d, "x")
     if x2d.dim() != 2 or x2d.shape[1] != in_tiles * 16:
@@ -590,6 +592,19 @@ def linear_forward(x2d, trellis, k, cb, suh=None, svh=None, bias=None, group_sub
         if member_out is None or len(member_out) != n_sub or sum(member_out) != n_out:
             raise ValueError("member_out must list the out_features of the stacked members")
         xh = had128_pre(x2d, suh)  # (rows, n_sub, in)
+        if all(n % 256 == 0 for n in member_out):
+            # members end on 256-column blocks: one GEMM launch over all of them, each
+            # block reading its member's rotation, then the output transform
+            if block_sub is None:
+                block_sub = group_sub[::2].contiguous()
+            lib = _lib.load()
+            ws_bytes = int(lib.exl3_linear_prefill_workspace_bytes(rows, n_in, n_out))
+            ws = workspace(x2d.device, ws_bytes)
+            rc = lib.exl3_linear_prefill(
+                _ptr(xh), rows, n_sub, _ptr(trellis), in_tiles, out_tiles, int(k), int(cb),
+                _ptr(block_sub), _ptr(svh), _ptr(bias), _ptr(y), _ptr(ws), ws.numel(), _stream())
+            _lib.check(rc, "exl3_linear_prefill")
+            return y
         tn0 = 0
         for i, n in enumerate(member_out):
             if n % 128:

@@ -243,3 +243,35 @@ def test_prefill_rows_with_every_tile_split(cuda, oracle, rows, k, n_in, n_out):
     assert rel_l2(y.cpu().numpy(), _oracle_forward(oracle, layer, x)) <= TOL
     parts = ops.had128_post(ops.inner_gemm(ops.had128_pre(xt, suh), tr, k, cb), svh, bias)
     assert torch.equal(y, parts)
+
+
+@pytest.mark.parametrize("rows", [17, 40, 300])
+def test_sibling_prefill_in_one_gemm_launch(cuda, oracle, rows):
+    """Members that end on 256-column blocks go through one GEMM launch in which
+    every block reads its own member's rotation; same result as member by member
+    (the path for members that do not end on block boundaries) and as the oracle."""
+    from ponyexl3_amd import FusedEXL3Group, make_exl3_layer, ops
+
+    layers = [make_exl3_layer(k=4, in_features=1024, out_features=o, seed=170 + i, mcg=True, key=f"s{i}")
+              for i, o in enumerate((512, 256, 256))]
+    group = FusedEXL3Group(layers)
+    assert group._block_sub is not None
+    rng = np.random.default_rng(rows)
+    x, xt = _x(rng, (rows, 1024), cuda)
+    print(f"sibling prefill rows={rows}", flush=True)
+    outs = group.forward_all(xt)
+    xh = ops.had128_pre(xt, group._suh_stack)
+    for i, (o, l) in enumerate(zip(outs, layers)):
+        assert rel_l2(o.cpu().numpy(), _oracle_forward(oracle, l, x)) <= TOL
+        member = ops.had128_post(ops.inner_gemm(xh[:, i].contiguous(), ops.as_trellis_tensor(l.trellis, cuda),
+                                                4, int(l.codebook_mode)),
+                                 torch.from_numpy(l.svh).to(cuda))
+        assert torch.equal(o, member)
+    # 384 columns: not a whole number of blocks -> member-by-member launches
+    odd_layers = [make_exl3_layer(k=4, in_features=512, out_features=o, seed=180 + i, key=f"o{i}")
+                  for i, o in enumerate((384, 128))]
+    odd = FusedEXL3Group(odd_layers)
+    assert odd._block_sub is None
+    x2, xt2 = _x(rng, (rows, 512), cuda)
+    for o, l in zip(odd.forward_all(xt2), odd_layers):
+        assert rel_l2(o.cpu().numpy(), _oracle_forward(oracle, l, x2)) <= TOL
