@@ -24,6 +24,25 @@ def codebook_mode_from_flags(mcg: bool = False, mul1: bool = False) -> CodebookM
     return CodebookMode.DEFAULT
 
 
+def tensor_core_perm() -> np.ndarray:
+    """Kernel order -> row-major position inside a 16x16 tile: ``kernel[i] =
+    row_major[perm[i]]`` (``tensor_core_perm``, ponyexl3/ref/perm.py:8-25). Closed
+    form: codewords 8t..8t+7 belong to the fragment lane t of an m16n8k16 B operand,
+    i.e. rows 2(t%4) + {0, 1, 8, 9} of columns t//4 and t//4 + 8."""
+    i = np.arange(256, dtype=np.int32)
+    t, j = i >> 3, i & 7
+    row = 2 * (t & 3) + (j & 1) + 8 * ((j >> 1) & 1)
+    col = (t >> 2) + 8 * (j >> 2)
+    return (row * 16 + col).astype(np.int32)
+
+
+def tensor_core_perm_inverse() -> np.ndarray:
+    """``row_major[p] = kernel[inv[p]]`` (ponyexl3/ref/perm.py:28-32)."""
+    inv = np.empty(256, dtype=np.int32)
+    inv[tensor_core_perm()] = np.arange(256, dtype=np.int32)
+    return inv
+
+
 def unpack_sign_bitfield(bitfield: np.ndarray) -> np.ndarray:
     """Packed int16 sign words (one per 16 channels, bit set = -1, least
     significant bit = first channel) -> +-1 float16."""

@@ -15,6 +15,7 @@ import numpy as np
 import torch
 
 from . import _lib
+from .layer import tensor_core_perm, tensor_core_perm_inverse
 from .ops import _check_cuda, _ptr, _stream
 
 # Bound on the backpointer scratch of one launch. The reference's default is
@@ -96,3 +97,53 @@ def pack_trellis(encoded, k: int, *, device="cuda") -> torch.Tensor:
         rc = _lib.load().exl3_pack_trellis(_ptr(arr), n_tiles, int(k), _ptr(out), _stream())
         _lib.check(rc, "exl3_pack_trellis")
     return out
+
+
+_perm_cache: dict = {}
+
+
+def _perm_tensors(device):
+    key = str(device)
+    if key not in _perm_cache:
+        _perm_cache[key] = (torch.from_numpy(tensor_core_perm().astype(np.int64)).to(device),
+                            torch.from_numpy(tensor_core_perm_inverse().astype(np.int64)).to(device))
+    return _perm_cache[key]
+
+
+def inner_to_kernel_tiles(inner: torch.Tensor) -> torch.Tensor:
+    """(in, out) matrix -> (in/16 * out/16, 256) fp32 tiles in kernel order, tiles
+    enumerated row-major over (tile row, tile column) (``_inner_to_kernel_tiles``,
+    ponyexl3/convert/direct.py:409-419)."""
+    if inner.dim() != 2 or inner.shape[0] % 16 or inner.shape[1] % 16:
+        raise ValueError(f"expected 2D matrix with 16-multiple dims, got {tuple(inner.shape)}")
+    tk, tn = inner.shape[0] // 16, inner.shape[1] // 16
+    perm, _ = _perm_tensors(inner.device)
+    row_major = inner.reshape(tk, 16, tn, 16).permute(0, 2, 1, 3).reshape(tk * tn, 256)
+    return row_major[:, perm].to(torch.float32).contiguous()
+
+
+def kernel_tiles_to_inner(tiles: torch.Tensor, rows: int, cols: int) -> torch.Tensor:
+    """Inverse of :func:`inner_to_kernel_tiles` (``_kernel_tiles_to_inner``,
+    ponyexl3/convert/direct.py:422-433)."""
+    tk, tn = rows // 16, cols // 16
+    if tuple(tiles.shape) != (tk * tn, 256):
+        raise ValueError(f"decoded tile shape {tuple(tiles.shape)} does not match {(rows, cols)}")
+    _, inv = _perm_tensors(tiles.device)
+    return tiles[:, inv].reshape(tk, tn, 16, 16).permute(0, 2, 1, 3).reshape(rows, cols).contiguous()
+
+
+def quantize_inner_matrix_direct(inner, *, k: int, cb: int = 0, return_states: bool = False,
+                                 max_scratch_bytes: int = DEFAULT_MAX_SCRATCH_BYTES, device="cuda"):
+    """Quantize an inner-domain matrix tile by tile, without LDL error feedback:
+    ``(packed trellis (in/16, out/16, 16K) int16, states or None, reconstructed (in,
+    out) fp32)``, all on the device (``quantize_inner_matrix_direct[_mlx]``,
+    ponyexl3/convert/direct.py:469-556). The packed trellis is what
+    ``exl3_decode_full`` and the forward kernels read."""
+    w = torch.as_tensor(inner, dtype=torch.float32, device=device)
+    tiles = inner_to_kernel_tiles(w)
+    q, idx = quantize_tiles(tiles, k, cb, max_scratch_bytes=max_scratch_bytes, device=w.device)
+    tk, tn = w.shape[0] // 16, w.shape[1] // 16
+    states = idx.reshape(tk, tn, 256)
+    packed = pack_trellis(states & ((1 << int(k)) - 1), k, device=w.device)
+    recon = kernel_tiles_to_inner(q, w.shape[0], w.shape[1])
+    return packed, (states if return_states else None), recon

@@ -135,3 +135,33 @@ def test_search_pack_decode_round_trip(cuda, oracle, k, cb):
     got = w_q.reshape(tk, 16, tn, 16).transpose(0, 2, 1, 3).reshape(tk * tn, 256)[:, perm]
     np.testing.assert_array_equal(got, q.cpu().numpy())
     assert float(np.mean((w_q - w) ** 2)) < 0.5 * float(np.mean(w ** 2))
+
+
+def test_quantize_inner_matrix_feeds_the_forward_kernels(cuda, oracle):
+    """Matrix in, trellis out: the packed result decodes (GPU and oracle) to the
+    reconstruction the search reports, and an EXL3Linear built on it multiplies by
+    exactly that matrix (no signs: suh = svh = 1)."""
+    from ponyexl3_amd import EXL3Layer, EXL3Linear, ops, search
+
+    rng = np.random.default_rng(11)
+    n_in, n_out, k = 128, 256, 4
+    w = (rng.standard_normal((n_in, n_out)) * 1.24).astype(np.float32)
+    packed, states, recon = search.quantize_inner_matrix_direct(w, k=k, cb=MCG, return_states=True, device=cuda)
+    assert tuple(packed.shape) == (n_in // 16, n_out // 16, 16 * k) and tuple(states.shape) == (8, 16, 256)
+    packed_np = packed.cpu().numpy().view(np.uint16)
+    np.testing.assert_array_equal(oracle.decode_trellis(packed_np, k, MCG).astype(np.float32), recon.cpu().numpy())
+    np.testing.assert_array_equal(ops.decode_full(packed, k, MCG).float().cpu().numpy(), recon.cpu().numpy())
+    tiles = search.inner_to_kernel_tiles(torch.from_numpy(w).to(cuda))
+    np.testing.assert_array_equal(search.kernel_tiles_to_inner(tiles, n_in, n_out).cpu().numpy(), w)
+    rel = float(np.linalg.norm(recon.cpu().numpy() - w) / np.linalg.norm(w))
+    assert rel < 0.1  # 4 bits per weight: about 7 % relative error on Gaussian weights
+    ones_in, ones_out = np.ones(n_in, np.float16), np.ones(n_out, np.float16)
+    layer = EXL3Layer("q", n_in, n_out, k, packed_np, ones_in, ones_out, None, mcg=True, mul1=False)
+    x = rng.standard_normal((3, n_in)).astype(np.float16)
+    y = EXL3Linear(layer)(torch.from_numpy(x).to(cuda)).cpu().numpy()
+    ref = oracle.linear_forward(packed_np, k, MCG, ones_in, ones_out, x)
+    np.testing.assert_allclose(y.astype(np.float32), ref.astype(np.float32), rtol=2e-3, atol=2e-2)
+    packed2, none_states, _ = search.quantize_inner_matrix_direct(w, k=k, cb=MCG, device=cuda)
+    assert none_states is None and torch.equal(packed2, packed)
+    with pytest.raises(ValueError):
+        search.quantize_inner_matrix_direct(np.zeros((100, 256), np.float32), k=4, device=cuda)

@@ -85,3 +85,14 @@ def test_ops_reject_cpu_tensors():
         ops.decode_full(torch.zeros((1, 1, 64), dtype=torch.int16), 4, 0)
     with pytest.raises(ValueError):
         ops.had128_pre(torch.zeros((1, 128), dtype=torch.float16), None)
+
+
+def test_tensor_core_perm_closed_form(oracle):
+    """The package's closed form equals the oracle's table (itself pinned by the
+    reference-written one) and is a bijection."""
+    from ponyexl3_amd.layer import tensor_core_perm, tensor_core_perm_inverse
+
+    perm = tensor_core_perm()
+    np.testing.assert_array_equal(perm, oracle.tensor_core_perm())
+    assert sorted(perm.tolist()) == list(range(256))
+    np.testing.assert_array_equal(perm[tensor_core_perm_inverse()], np.arange(256))
