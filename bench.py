@@ -299,7 +299,8 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f16 weights decoded from K-bit trellis codes, f32 accumulate",
+        "dtype": "f16",
+        "dtype_note": "K-bit trellis codes decoded to f16 weights (u32 integer decode), f16 activations, f32 accumulate",
         "data": "synthetic (seeded random trellis words, +-1 signs, N(0,1) fp16 activations)",
         "config": {
             "workload": "configs[1]: 27B-class dense decoder linears at batch 1, K=4, 3INST; "
