@@ -98,6 +98,9 @@ __global__ __launch_bounds__(256, 2) void quantize_tiles_kernel(const float* __r
     const uint32_t low = (uint32_t)tid & (KK - 1);
     const uint32_t base = ((uint32_t)tid >> K) * PER_LANE;  // e(j) >> K = base + j
     uint16_t* back = back_ws + (size_t)blockIdx.x * 256 * EDGES;
+    // lane parts of the cost-row addresses (see unit_addr and the store below)
+    const uint32_t lane_rd0 = KR - K >= 8 ? base + (base >> 8) * PAD : base;
+    const uint32_t lane_wr0 = row_index((base << K) | low);
 
     // decoded values of the lane's codewords, index c = f*PER_LANE + j, two per register
     half2_t lut[128];
@@ -135,7 +138,6 @@ __global__ __launch_bounds__(256, 2) void quantize_tiles_kernel(const float* __r
                 const half_t* cprev = costs + ((step & 1) ^ 1) * ROW;
                 half_t* ccurr = costs + (step & 1) * ROW;
                 const float negt = -target_s[ri];
-                const bool keep = pass == 1 || ri < 128;
                 // The table is the same in every step; without this the compiler hoists
                 // its 256 fp16 -> fp32 conversions out of the loop and runs out of registers.
 #pragma unroll
@@ -148,13 +150,18 @@ __global__ __launch_bounds__(256, 2) void quantize_tiles_kernel(const float* __r
                 constexpr bool ALONG_F = PER_LANE == 1;
                 constexpr int UNIT = ALONG_F ? 8 : CH;
                 constexpr int N_UNITS = 256 / UNIT;
+                // Address = lane part (computed once) + a compile-time part that fits the
+                // immediate offset of the LDS instruction. The split is exact: the fresh
+                // value contributes whole 256-state blocks (K <= 4) or decides the block
+                // on its own (K > 4), and a lane's states never cross a block.
                 auto unit_addr = [&](int u) -> const half_t* {
                     if constexpr (ALONG_F) {
                         return cprev + u * 8;  // base = 0: predecessor = fresh
                     } else {
                         const int ch = u / KK, f = u % KK;
-                        // the lane's states of one chunk lie inside one block of 256
-                        return cprev + row_index(((uint32_t)f << (KR - K)) | (base + ch * CH));
+                        const int fpart = f << (KR - K);
+                        const int blocks = KR - K >= 8 ? fpart >> 8 : f >> (8 - (KR - K));
+                        return cprev + lane_rd0 + (fpart + ch * CH + blocks * PAD);
                     }
                 };
                 auto fetch = [&](int u) {
@@ -227,17 +234,25 @@ __global__ __launch_bounds__(256, 2) void quantize_tiles_kernel(const float* __r
                         }
                     }
                     if constexpr (f_last == KK - 1) {
+                        // one scalar base per chunk; the stores below differ only in their
+                        // immediate offsets and share the lane offset (otherwise the compiler
+                        // keeps a separate offset register per store, 64 of them at K = 2)
+                        size_t row_off = (size_t)ri * EDGES + (ch * CH) * 256;
+                        asm volatile("" : "+s"(row_off));
+                        uint16_t* rowbase = back + row_off;
 #pragma unroll
                         for (int b = 0; b < NB; b++) {
                             const uint32_t pj = base + ch * CH + b;
-                            const uint32_t e = (pj << K) | low;
-                            ccurr[row_index(e)] = (half_t)best[b];
-                            if (keep) {
-                                // the reference leaves the backpointer at 0 when nothing beat the bound
-                                const uint32_t bp =
-                                    best_f[b] == kNoneAll ? 0u : (best_f[b] << (KR - K)) | pj;
-                                back[(size_t)ri * EDGES + (ch * CH + b) * 256 + tid] = (uint16_t)bp;
-                            }
+                            // state (pj << K) | low: all states of a lane lie in one block
+                            ccurr[lane_wr0 + ((ch * CH + b) << K)] = (half_t)best[b];
+                            // The reference leaves the backpointer at 0 when nothing beat the
+                            // bound. It skips the store for positions 128..255 of the warm-up
+                            // pass, which nobody reads; storing them anyway (the pinned pass
+                            // rewrites every row before it is walked) keeps the loop free of
+                            // branches.
+                            const uint32_t bp =
+                                best_f[b] == kNoneAll ? 0u : (best_f[b] << (KR - K)) | pj;
+                            rowbase[b * 256 + tid] = (uint16_t)bp;
                         }
                     }
                     cur = nxt;
@@ -316,15 +331,15 @@ __global__ __launch_bounds__(256) void pack_trellis_kernel(const uint16_t* __res
 }
 
 // Workgroups the search keeps resident: the kernel holds its decode table in
-// registers and is compiled for two waves per SIMD, i.e. two workgroups per CU.
+// registers; its register count leaves room for two waves per SIMD, i.e. two
+// workgroups per CU (three from K = 6 on, where fewer address registers are live).
 static int quantize_slots_wanted(int K) {
-    (void)K;
     hipDeviceProp_t prop;
     int dev = 0;
     int cus = 256;
     if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
         cus = prop.multiProcessorCount;
-    return cus * 2;
+    return cus * (K >= 6 ? 3 : 2);
 }
 
 }  // namespace exl3
