@@ -119,14 +119,30 @@ def cpu_baseline(budget_s=12.0):
             c0 += n_out
     x = {n: np.random.default_rng(n).standard_normal(n).astype(np.float16) for n in (5120, 8192, 17408)}
     total = sum(weight_bytes(n_in, outs) for _, n_in, outs in LAYER)
-    reps, t0 = 0, time.perf_counter()
-    while True:
-        for tr, suh, svh, n_in in layers:
-            orc.linear_forward_bs1(tr, K_BITS, CB, suh, svh, x[n_in])
-        reps += 1
-        dt = time.perf_counter() - t0
-        if dt > budget_s:
-            break
+
+    def run(seconds):
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            for tr, suh, svh, n_in in layers:
+                orc.linear_forward_bs1(tr, K_BITS, CB, suh, svh, x[n_in])
+            reps += 1
+            dt = time.perf_counter() - t0
+            if dt > seconds:
+                return reps, dt
+
+    reps, dt = run(budget_s)
+    orc.set_num_threads(1)  # one pass on a single core for scale (about 4 s)
+    reps1, dt1 = run(0.0)
+    orc.set_num_threads(threads)
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo", encoding="utf-8") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
     return {
         "value": round(total * reps / dt / 1e9, 4),
         "unit": "GB/s",
@@ -135,6 +151,8 @@ def cpu_baseline(budget_s=12.0):
         "sample": f"{reps} pass(es) over one config-2 decoder layer at batch 1 "
                   f"({total / 1e6:.1f} MB of K=4 trellis, decode + Hadamard-128 + matvec), "
                   f"C oracle with OpenMP, {dt:.1f} s",
+        "single_core_value": round(total * reps1 / dt1 / 1e9, 4),
+        "cpu_model": model,
     }
 
 
