@@ -312,6 +312,15 @@ int exl3_moe_glu_rows(const uint16_t *g, const uint16_t *u, int n_rows, int H, c
                       int activation, uint16_t *xh_dn, void *stream);
 
 /*
+ * Packed tiles -> their 256 sliding-window codewords per tile, kernel order.
+ * Replaces unpack_trellis (ponyexl3/ref/trellis.py:153-214); the inverse of
+ * exl3_pack_trellis on the low K bits. K in 1..8.
+ *   trellis u16 [n_tiles][16*K]   codewords u16 [n_tiles][256] (16-byte aligned)
+ */
+int exl3_unpack_trellis(const uint16_t *trellis, long long n_tiles, int K, uint16_t *codewords,
+                        void *stream);
+
+/*
  * Encoder side: tail-biting Viterbi search over the bitshift trellis, one 16x16
  * tile (256 fp32 targets in kernel order) per workgroup. Replaces
  * quantize_tiles_mlx (ponyexl3/convert/metal_search.py:63-196, 254-303) and

@@ -41,6 +41,7 @@ PROTOTYPES = {
     "exl3_quantize_slot_bytes": (_sz, [_i]),
     "exl3_quantize_workspace_bytes": (_sz, [_i, _i]),
     "exl3_quantize_tiles": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _sz, _vp]),
+    "exl3_unpack_trellis": (_i, [_vp, ctypes.c_longlong, _i, _vp, _vp]),
     "exl3_pack_trellis": (_i, [_vp, ctypes.c_longlong, _i, _vp, _vp]),
     "exl3_decode_full_eg": (_i, [_vp, _i, _i, _i, _i, _i, _vp, _vp]),
     "exl3_decode_full_t": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _vp]),

@@ -116,6 +116,35 @@ __global__ __launch_bounds__(256) void decode_full_t_kernel(const uint32_t* __re
     }
 }
 
+// Packed tiles -> their 256 16-bit codewords in kernel (stream) order
+// (unpack_trellis, ponyexl3/ref/trellis.py:153-214). Lanes 8t..8t+7 of a wave own
+// tile t of eight consecutive tiles; lane u extracts codewords 32u..32u+31 and
+// writes them as 64 contiguous bytes.
+template <int K>
+__global__ __launch_bounds__(256) void unpack_trellis_kernel(const uint32_t* __restrict__ trellis,
+                                                             uint16_t* __restrict__ codewords,
+                                                             long long n_tiles) {
+    const int lane = threadIdx.x & 63;
+    const long long wid = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const long long tile_lane = wid * 8 + (lane >> 3);
+    // lanes past the last tile re-read it (never stored)
+    const long long tile = tile_lane < n_tiles ? tile_lane : n_tiles - 1;
+    const uint32_t* p = trellis + tile * (8 * K) + (lane & 7) * K;
+    uint32_t own[K];
+#pragma unroll
+    for (int i = 0; i < K; i++) own[i] = p[i];
+    const LaneWords<K> lw = finish_lane_words<K>(own, lane);
+    uint32_t packed[16];
+    static_for<0, 16>([&](auto i) {
+        packed[i.value] = lane_codeword<K, 2 * i.value>(lw) | (lane_codeword<K, 2 * i.value + 1>(lw) << 16);
+    });
+    if (tile_lane >= n_tiles) return;
+    uint4_t* dst = reinterpret_cast<uint4_t*>(codewords + tile * 256 + (lane & 7) * 32);
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        dst[i] = uint4_t{packed[4 * i], packed[4 * i + 1], packed[4 * i + 2], packed[4 * i + 3]};
+}
+
 // Shared argument checks and launch of the row-major / expert-grouped kernel.
 static int launch_decode_full(const uint16_t* trellis, int in_tiles, int out_tiles, int K, int cb,
                               int tn_offset, int tn_count, int tiles_per_group, uint16_t* w_out,
@@ -175,6 +204,24 @@ EXL3_EXPORT int exl3_decode_full_t(const uint16_t* trellis, int in_tiles, int ou
             <<<dim3((unsigned)grid), dim3(256), 0, as_stream(stream)>>>(
                 reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<half_t*>(w_out_t),
                 in_tiles, out_tiles, tn_offset, tn_count);
+        return launch_status();
+    });
+}
+
+EXL3_EXPORT int exl3_unpack_trellis(const uint16_t* trellis, long long n_tiles, int K,
+                                    uint16_t* codewords, void* stream) {
+    using namespace exl3;
+    if (K < 1 || K > 8) return EXL3_E_BAD_K;
+    if (n_tiles < 0) return EXL3_E_BAD_SHAPE;
+    if (n_tiles == 0) return EXL3_OK;
+    if (!trellis || !codewords) return EXL3_E_NULL_POINTER;
+    if ((reinterpret_cast<uintptr_t>(trellis) & 3) || (reinterpret_cast<uintptr_t>(codewords) & 15))
+        return EXL3_E_BAD_SHAPE;
+    const long long grid = (n_tiles + 31) / 32;
+    if (grid > 0x7FFFFFFFLL) return EXL3_E_BAD_SHAPE;
+    return dispatch_k_cb(K, 0, [&](auto k, auto) {
+        unpack_trellis_kernel<k.value><<<dim3((unsigned)grid), dim3(256), 0, as_stream(stream)>>>(
+            reinterpret_cast<const uint32_t*>(trellis), codewords, n_tiles);
         return launch_status();
     });
 }

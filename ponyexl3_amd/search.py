@@ -99,6 +99,30 @@ def pack_trellis(encoded, k: int, *, device="cuda") -> torch.Tensor:
     return out
 
 
+def unpack_trellis(packed, k: int, *, device="cuda") -> torch.Tensor:
+    """Packed ``(..., 16*K)`` trellis words -> ``(..., 256)`` 16-bit codewords in
+    kernel order (int16 storage of the uint16 bits); ``unpack_trellis``,
+    ponyexl3/ref/trellis.py:153-214. The low K bits are what :func:`pack_trellis`
+    takes."""
+    if not 1 <= int(k) <= 8:
+        raise ValueError(f"K must be in [1, 8], got {k}")
+    if isinstance(packed, np.ndarray):
+        packed = torch.from_numpy(np.ascontiguousarray(packed).astype(np.uint16).view(np.int16))
+    arr = packed.to(device)
+    if arr.dtype == torch.uint16:
+        arr = arr.view(torch.int16)
+    if arr.dtype != torch.int16 or arr.dim() < 1 or arr.shape[-1] != 16 * int(k):
+        raise ValueError(f"expected 16-bit words with last dim {16 * int(k)}, got {arr.dtype} {tuple(arr.shape)}")
+    arr = arr.contiguous()
+    _check_cuda(arr, "packed")
+    out = torch.empty(tuple(arr.shape[:-1]) + (256,), dtype=torch.int16, device=arr.device)
+    n_tiles = out.numel() // 256
+    if n_tiles:
+        rc = _lib.load().exl3_unpack_trellis(_ptr(arr), n_tiles, int(k), _ptr(out), _stream())
+        _lib.check(rc, "exl3_unpack_trellis")
+    return out
+
+
 _perm_cache: dict = {}
 
 
@@ -133,6 +157,7 @@ def kernel_tiles_to_inner(tiles: torch.Tensor, rows: int, cols: int) -> torch.Te
 
 
 def quantize_inner_matrix_direct(inner, *, k: int, cb: int = 0, return_states: bool = False,
+                                 verify_roundtrip: bool = False,
                                  max_scratch_bytes: int = DEFAULT_MAX_SCRATCH_BYTES, device="cuda"):
     """Quantize an inner-domain matrix tile by tile, without LDL error feedback:
     ``(packed trellis (in/16, out/16, 16K) int16, states or None, reconstructed (in,
@@ -145,5 +170,7 @@ def quantize_inner_matrix_direct(inner, *, k: int, cb: int = 0, return_states: b
     tk, tn = w.shape[0] // 16, w.shape[1] // 16
     states = idx.reshape(tk, tn, 256)
     packed = pack_trellis(states & ((1 << int(k)) - 1), k, device=w.device)
+    if verify_roundtrip and not torch.equal(unpack_trellis(packed, k, device=w.device), states):
+        raise AssertionError("direct quantization produced non-round-trippable trellis")
     recon = kernel_tiles_to_inner(q, w.shape[0], w.shape[1])
     return packed, (states if return_states else None), recon

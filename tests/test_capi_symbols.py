@@ -63,6 +63,9 @@ def test_argument_errors_before_launch(lib):
     assert lib.exl3_pack_trellis(p, 1, 0, p, None) == _lib.EXL3_E_BAD_K
     assert lib.exl3_pack_trellis(p, 1, 4, None, None) == _lib.EXL3_E_NULL_POINTER
     assert lib.exl3_pack_trellis(p, 0, 4, p, None) == _lib.EXL3_OK
+    assert lib.exl3_unpack_trellis(p, 1, 9, p, None) == _lib.EXL3_E_BAD_K
+    assert lib.exl3_unpack_trellis(None, 1, 4, p, None) == _lib.EXL3_E_NULL_POINTER
+    assert lib.exl3_unpack_trellis(p, 0, 4, p, None) == _lib.EXL3_OK
     assert lib.exl3_linear_prefill(p, 4, 2, p, 8, 16, 4, 0, None, p, None, p, p, 1 << 30, None) == _lib.EXL3_E_BAD_INDEX
     assert lib.exl3_linear_prefill(p, 4, 1, p, 8, 16, 4, 0, None, p, None, p, p, 16, None) == _lib.EXL3_E_WORKSPACE
     assert lib.exl3_linear_prefill(p, 4, 1, p, 7, 16, 4, 0, None, p, None, p, p, 1 << 30, None) == _lib.EXL3_E_BAD_SHAPE

@@ -161,7 +161,26 @@ def test_quantize_inner_matrix_feeds_the_forward_kernels(cuda, oracle):
     y = EXL3Linear(layer)(torch.from_numpy(x).to(cuda)).cpu().numpy()
     ref = oracle.linear_forward(packed_np, k, MCG, ones_in, ones_out, x)
     np.testing.assert_allclose(y.astype(np.float32), ref.astype(np.float32), rtol=2e-3, atol=2e-2)
-    packed2, none_states, _ = search.quantize_inner_matrix_direct(w, k=k, cb=MCG, device=cuda)
+    packed2, none_states, _ = search.quantize_inner_matrix_direct(w, k=k, cb=MCG, device=cuda,
+                                                                  verify_roundtrip=True)
     assert none_states is None and torch.equal(packed2, packed)
     with pytest.raises(ValueError):
         search.quantize_inner_matrix_direct(np.zeros((100, 256), np.float32), k=4, device=cuda)
+
+
+@pytest.mark.parametrize("k", [1, 2, 3, 4, 5, 6, 7, 8])
+def test_unpack_trellis_bit_exact(cuda, oracle, k):
+    """Raw random words (every fill is a legal bitstream), 37 tiles = a partly filled
+    last wavefront: codewords equal the oracle's unpack; pack(unpack & mask) is the
+    identity."""
+    from ponyexl3_amd import search
+
+    rng = np.random.default_rng(500 + k)
+    packed = rng.integers(0, 65536, size=(37, 16 * k), dtype=np.uint16)
+    got = search.unpack_trellis(packed, k, device=cuda)
+    ref = np.stack([oracle.unpack_tile(t, k) for t in packed])
+    np.testing.assert_array_equal(got.cpu().numpy().view(np.uint16), ref)
+    again = search.pack_trellis(got & ((1 << k) - 1), k, device=cuda)
+    np.testing.assert_array_equal(again.cpu().numpy().view(np.uint16), packed)
+    with pytest.raises(ValueError):
+        search.unpack_trellis(packed, k % 8 + 1, device=cuda)
