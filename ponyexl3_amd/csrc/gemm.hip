@@ -51,16 +51,42 @@ struct GemmWork {
     int tile, k_begin, k_end, partial_unit;  // partial_unit < 0: direct fp16 output
 };
 
+// Workgroups are handed to the eight XCDs round-robin by index, and each XCD has
+// its own L2. Whole tiles are numbered column block first (tile = g * n_row_blocks
+// + row block), so consecutive indices would spread the row blocks of one column
+// block -- which all decode the same trellis columns -- over all eight L2s. For the
+// part of the schedule that holds complete sets of eight column blocks, workgroup b
+// therefore takes column block 8*(q / n_row_blocks) + b % 8, row block q %
+// n_row_blocks with q = b / 8: a column block stays on one XCD.
+__device__ __forceinline__ int xcd_tile_order(int b, int full_tiles, int n_row_blocks) {
+    const int set = 8 * n_row_blocks;
+    const int whole = full_tiles / set * set;
+    if (b >= whole) return b;
+    const int q = b >> 3;
+    const int g = (q / n_row_blocks) * 8 + (b & 7);
+    return g * n_row_blocks + q % n_row_blocks;
+}
+
 __device__ __forceinline__ GemmWork gemm_work(int unit, int full_tiles, int split,
-                                              int ksteps_per_split, int ksteps) {
+                                              int ksteps_per_split, int ksteps,
+                                              int n_row_blocks, int split_units) {
     GemmWork w;
     if (unit < full_tiles) {
-        w.tile = unit;
+        w.tile = xcd_tile_order(unit, full_tiles, n_row_blocks);
         w.k_begin = 0;
         w.k_end = ksteps;
         w.partial_unit = -1;
     } else {
-        const int r = unit - full_tiles;
+        // Split tiles: the units that share trellis data are the row blocks of one
+        // (column block, reduction range) pair. Those pairs are numbered gv = column
+        // block * split + range, units v = gv * n_row_blocks + row block, and v is
+        // dealt to the XCDs like the whole tiles above.
+        int r = unit - full_tiles;  // canonical index: (tile - full_tiles) * split + range
+        if (full_tiles % n_row_blocks == 0) {
+            const int v = xcd_tile_order(r, split_units, n_row_blocks);
+            const int gv = v / n_row_blocks, rb = v % n_row_blocks;
+            r = ((gv / split) * n_row_blocks + rb) * split + gv % split;
+        }
         w.tile = full_tiles + r / split;
         const int sp = r % split;
         w.k_begin = sp * ksteps_per_split;
@@ -106,7 +132,8 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
         tn_offset = tn_offset_arg + t.x * group_tiles;
         tn_count = group_tiles;
     } else {
-        work = gemm_work(blockIdx.x, full_tiles, split, ksteps_per_split, in_tiles / 4);
+        work = gemm_work(blockIdx.x, full_tiles, split, ksteps_per_split, in_tiles / 4,
+                         n_row_blocks, (int)gridDim.x - full_tiles);
         g = work.tile / n_row_blocks;  // 256-column block inside the slice
         m0 = (work.tile % n_row_blocks) * BM;
         rows = rows_arg;
