@@ -111,3 +111,16 @@ def test_status_to_exception():
         _lib.check(_lib.EXL3_E_BAD_SHAPE, "x")
     with pytest.raises(RuntimeError):
         _lib.check(_lib.EXL3_E_LAUNCH, "x")
+
+
+def test_header_is_plain_c_and_cxx():
+    """include/exl3_hip.h is the boundary: it has to compile on its own as C99 and as
+    C++ (no HIP or torch types in any signature)."""
+    import shutil
+    import subprocess
+
+    header = os.path.join(ROOT, "include", "exl3_hip.h")
+    if shutil.which("gcc") is None:
+        pytest.skip("gcc not available")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-fsyntax-only", "-x", "c", header], check=True)
+    subprocess.run(["g++", "-std=c++17", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", header], check=True)
