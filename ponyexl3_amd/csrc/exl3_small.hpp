@@ -50,7 +50,11 @@ __device__ __forceinline__ void wht128_lanes(float& a, float& b, int lane) {
 // The raw block after the current one is in flight while the current one is
 // used; a tile row's 16 activations come back with two broadcast ds_read_b128.
 // kSlots wave-wide trellis loads are kept in flight.
-template <int K, int CB, int MT, bool ROTATE>
+//
+// HALF: the range is one half of a block, [tk_begin, tk_begin + 4) with tk_begin a
+// multiple of 4. The wave still rotates (or stages) the whole 128-wide block, then
+// uses four of its eight tile rows. Narrow layers get twice the waves this way.
+template <int K, int CB, int MT, bool ROTATE, bool HALF = false>
 __device__ __forceinline__ void stream_block_rows(const uint32_t* __restrict__ base,
                                                   size_t row_words, int tk_begin, int tk_end,
                                                   const half_t* __restrict__ x, size_t x_stride,
@@ -138,10 +142,36 @@ __device__ __forceinline__ void stream_block_rows(const uint32_t* __restrict__ b
             }
         }
     };
-    // Ranges are whole blocks, so the staging sits outside the unrolled 8-step
-    // pipeline and the LDS offsets of the activations are compile-time constants.
     constexpr int kSlots = 4;  // wave-wide loads in flight (divides the 8 steps of a block)
     uint32_t buf[kSlots][K];
+    if constexpr (HALF) {
+        // all four loads up front, no refills
+#pragma unroll
+        for (int s = 0; s < kSlots; s++)
+            load_lane_words_nt<K>(base + (size_t)(tk_begin + s) * row_words, buf[s]);
+        fetch_block(tk_begin >> 3);
+        stage_block();
+        const int row0 = tk_begin & 7;  // 0 or 4
+        uint32_t prev = neighbour_word(buf[0][K - 1], lane);
+#pragma unroll
+        for (int s = 0; s < kSlots; s++) {
+            const uint32_t prev_next =
+                s + 1 < kSlots ? neighbour_word(buf[s + 1][K - 1], lane) : 0u;
+            const XTile xt = load_x(row0 + s);
+            __builtin_amdgcn_sched_barrier(0);
+            consume(buf[s], prev, xt);
+            __builtin_amdgcn_sched_barrier(0);
+            prev = prev_next;
+        }
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            acc[m][0] += accv[0][m >> 2][m & 3];
+            acc[m][1] += accv[1][m >> 2][m & 3];
+        }
+        return;
+    }
+    // Ranges are whole blocks, so the staging sits outside the unrolled 8-step
+    // pipeline and the LDS offsets of the activations are compile-time constants.
 #pragma unroll
     for (int s = 0; s < kSlots; s++)
         load_lane_words_nt<K>(base + (size_t)min(tk_begin + s, tk_end - 1) * row_words, buf[s]);

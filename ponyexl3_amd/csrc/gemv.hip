@@ -189,7 +189,8 @@ __global__ __launch_bounds__(256) void gemv_kernel(
 // input transform per sibling done by the Hadamard kernel; the waves only stage
 // it. Rotating sixteen rows in every workgroup would cost more instructions than
 // the decode itself.
-template <int K, int CB, int MT, bool ROTATE>
+// HALF (one and two rows only): splits are half blocks of four tile rows.
+template <int K, int CB, int MT, bool ROTATE, bool HALF>
 __global__ __launch_bounds__(256) void linear_small_kernel(
     const uint32_t* __restrict__ trellis, const half_t* __restrict__ x,
     const half_t* __restrict__ suh, const half_t* __restrict__ svh,
@@ -204,7 +205,7 @@ __global__ __launch_bounds__(256) void linear_small_kernel(
     const bool active = split < n_splits;  // idle waves still take part in the barriers below
     const int sub = group_sub ? group_sub[g] : 0;
     const int in_features = in_tiles * 16;
-    const int tk_begin = active ? split * tk_per_split : 0;  // tk_per_split is a multiple of 8
+    const int tk_begin = active ? split * tk_per_split : 0;  // tk_per_split: multiple of 8, or 4 (HALF)
     const int tk_end = active ? min(in_tiles, tk_begin + tk_per_split) : 0;
     const size_t row_words = (size_t)out_tiles * (8 * K);
     const uint32_t* base = trellis + (size_t)g * 8 * (8 * K) + lane * K;
@@ -218,8 +219,8 @@ __global__ __launch_bounds__(256) void linear_small_kernel(
 
     // ---- input Hadamard (or staging) + decode/dot pipeline over this wave's blocks
     if (active)
-        stream_block_rows<K, CB, MT, ROTATE>(base, row_words, tk_begin, tk_end, x_rows, x_stride,
-                                             rows, suh_row, xs[wave], lane, acc);
+        stream_block_rows<K, CB, MT, ROTATE, HALF>(base, row_words, tk_begin, tk_end, x_rows,
+                                                   x_stride, rows, suh_row, xs[wave], lane, acc);
 
     // ---- the four waves of the workgroup are summed through LDS in wave order,
     // the workgroup stores ONE fp32 partial row, and the last workgroup of the
@@ -354,10 +355,16 @@ GemvPlan plan_gemv(int rows, int in_tiles, int n_groups) {
 // Plan of the one-launch layer kernel: splits are whole Hadamard blocks (8 tile
 // rows) and every wave gets the same number of blocks where that divides.
 GemvPlan plan_linear_small(int rows, int in_tiles, int n_groups) {
-    (void)rows;
     static const int kWavesPerSimd = env_int("EXL3_LINEAR_WAVES_PER_SIMD", 12, 1, 16);
+    // one and two rows: when even one block per wave leaves fewer than this many waves
+    // (four per SIMD), the waves take half blocks
+    static const int kHalfBelow = env_int("EXL3_LINEAR_HALF_BELOW", 4096, 0, 1 << 20);
     const int target_waves = 256 * 4 * kWavesPerSimd;
     const int n_blocks = in_tiles / 8;
+    // (not with more than 48 blocks: 100+ partial rows per column group cost the
+    // finishing workgroup more than the extra waves gain; measured on 8192 -> 5120)
+    if (rows <= 2 && n_blocks <= 48 && (long long)n_blocks * n_groups < kHalfBelow)
+        return GemvPlan{n_blocks * 2, 4};
     int max_splits = target_waves / (n_groups > 0 ? n_groups : 1);
     if (max_splits < 1) max_splits = 1;
     if (max_splits > n_blocks) max_splits = n_blocks;
@@ -414,15 +421,17 @@ int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, in
     // variant for the row counts above that
     if (pre_rotated != (rows > kGemvMaxRows)) return EXL3_E_UNSUPPORTED;
     if (n_sub > 1 && (!group_sub || (!suh && !pre_rotated))) return EXL3_E_BAD_INDEX;
-    if (plan.n_splits < 1 || plan.n_splits > 4 * 65535 || plan.tk_per_split < 8 ||
-        plan.tk_per_split % 8 || (long long)plan.n_splits * plan.tk_per_split < in_tiles)
+    const bool half = plan.tk_per_split == 4 && rows <= 2;
+    if (plan.n_splits < 1 || plan.n_splits > 4 * 65535 ||
+        (!half && (plan.tk_per_split < 8 || plan.tk_per_split % 8)) ||
+        (long long)plan.n_splits * plan.tk_per_split < in_tiles)
         return EXL3_E_BAD_SHAPE;
     const int n_groups = out_tiles / 8;
     const dim3 grid((unsigned)n_groups, (unsigned)((plan.n_splits + 3) / 4));
     const int mt = rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : rows <= 8 ? 8 : 16;
     return dispatch_k_cb(K, cb, [&](auto k, auto c) {
-        auto go = [&](auto mtc, auto rot) {
-            linear_small_kernel<k.value, c.value, mtc.value, rot.value>
+        auto go = [&](auto mtc, auto rot, auto halfc) {
+            linear_small_kernel<k.value, c.value, mtc.value, rot.value, halfc.value>
                 <<<grid, dim3(256), 0, stream>>>(
                     reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<const half_t*>(x),
                     reinterpret_cast<const half_t*>(suh), reinterpret_cast<const half_t*>(svh),
@@ -430,12 +439,20 @@ int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, in
                     counters, group_sub, in_tiles, out_tiles, rows, n_groups, plan.tk_per_split,
                     plan.n_splits, n_sub);
         };
+        using T = std::true_type;
+        using F = std::false_type;
         switch (mt) {
-            case 1: go(std::integral_constant<int, 1>{}, std::true_type{}); break;
-            case 2: go(std::integral_constant<int, 2>{}, std::true_type{}); break;
-            case 4: go(std::integral_constant<int, 4>{}, std::true_type{}); break;
-            case 8: go(std::integral_constant<int, 8>{}, std::true_type{}); break;
-            default: go(std::integral_constant<int, 16>{}, std::false_type{}); break;
+            case 1:
+                if (half) go(std::integral_constant<int, 1>{}, T{}, T{});
+                else go(std::integral_constant<int, 1>{}, T{}, F{});
+                break;
+            case 2:
+                if (half) go(std::integral_constant<int, 2>{}, T{}, T{});
+                else go(std::integral_constant<int, 2>{}, T{}, F{});
+                break;
+            case 4: go(std::integral_constant<int, 4>{}, T{}, F{}); break;
+            case 8: go(std::integral_constant<int, 8>{}, T{}, F{}); break;
+            default: go(std::integral_constant<int, 16>{}, F{}, F{}); break;
         }
         return launch_status();
     });
