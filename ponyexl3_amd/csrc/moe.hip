@@ -14,6 +14,8 @@
 //                           128-column group of gate/up)
 //   B. moe_down_kernel      per (slot, 128 columns of D): decode GEMV over H on
 //                           the rotated block, sum, post-Hadamard, svh
+//   (four waves per workgroup, one Hadamard block of the reduction each; with few
+//   slots eight waves on half a block each, which doubles the loads in flight)
 // Without counters the same result comes from a chain of five launches:
 //   1. moe_prep_kernel      rotated activations per (slot, proj) + group tables
 //   2. gemv_kernel          gate/up partial sums, fp32
@@ -30,6 +32,7 @@
 #include "exl3_small.hpp"
 
 #include <algorithm>
+#include <type_traits>
 
 #pragma clang fp contract(off)
 
@@ -159,19 +162,22 @@ __global__ __launch_bounds__(256) void moe_finish_kernel(
 
 
 // ---------------------------------------------------------------------------
-// Fused chain: shared tail of both kernels. The four waves of a workgroup are
+// Fused chain: shared tail of both kernels. The NW waves of a workgroup are
 // added through LDS in wave order; returns the two sums of this lane's columns
 // (2*lane, 2*lane+1) to wave 0.
+template <int NW>
 __device__ __forceinline__ float2_t moe_wg_sum(float (*red)[128], const float (&acc)[1][2],
                                                int lane, int wave) {
     const int c0 = (lane >> 3) * 16 + (lane & 7);
     red[wave][c0] = acc[0][0];
     red[wave][c0 + 8] = acc[0][1];
     __syncthreads();
-    float2_t v;
-    v.x = ((red[0][2 * lane] + red[1][2 * lane]) + red[2][2 * lane]) + red[3][2 * lane];
-    v.y = ((red[0][2 * lane + 1] + red[1][2 * lane + 1]) + red[2][2 * lane + 1]) +
-          red[3][2 * lane + 1];
+    float2_t v{red[0][2 * lane], red[0][2 * lane + 1]};
+#pragma unroll
+    for (int w = 1; w < NW; w++) {
+        v.x = __fadd_rn(v.x, red[w][2 * lane]);
+        v.y = __fadd_rn(v.y, red[w][2 * lane + 1]);
+    }
     return v;
 }
 
@@ -216,14 +222,14 @@ __device__ __forceinline__ void moe_finish_block(float2_t sum, half2_t sv, int l
 // the Hadamard block 4q + w of D for slot s = gid / (2*hblocks), projection
 // p = (gid / hblocks) & 1 and column block hg = gid % hblocks.
 // part: fp32 [gid][n_wg][128]; counters[s*hblocks + hg] count 2*n_wg workgroups.
-template <int K, int CB>
-__global__ __launch_bounds__(256) void moe_gateup_kernel(
+template <int K, int CB, int NW>
+__global__ __launch_bounds__(NW * 64) void moe_gateup_kernel(
     const uint32_t* __restrict__ gu_trellis, const half_t* __restrict__ x,
     const int* __restrict__ indices, const half_t* __restrict__ gu_suh,
     const half_t* __restrict__ gu_svh, const half_t* __restrict__ dn_suh, half_t* xh_dn,
     float* part, int* counters, int top_k, int E, int D, int H, int activation) {
-    __shared__ __attribute__((aligned(16))) half_t xs[4][1][kXwLd];
-    __shared__ float red[4][128];
+    __shared__ __attribute__((aligned(16))) half_t xs[NW][1][kXwLd];
+    __shared__ float red[NW][128];
     __shared__ float up_val[128];
     __shared__ int last_flag;
     const int lane = threadIdx.x & 63;
@@ -234,17 +240,21 @@ __global__ __launch_bounds__(256) void moe_gateup_kernel(
     const int hg = gid % hblocks, sp = gid / hblocks;
     const int s = sp >> 1, p = sp & 1;
     const int e = clamp_expert(indices[s], E);
-    const int blk = blockIdx.y * 4 + wave;
+    constexpr bool kHalf = NW == 8;
+    const int part_idx = blockIdx.y * NW + wave;
+    const int blk = kHalf ? part_idx >> 1 : part_idx;
+    const int tk0 = blk * 8 + (kHalf ? (part_idx & 1) * 4 : 0);
     float acc[1][2] = {{0.f, 0.f}};
     if (blk < dblocks) {
         const size_t row_words = (size_t)E * 2 * (H >> 4) * (8 * K);
         const uint32_t* base =
             gu_trellis + ((size_t)(p * E + e) * (H >> 4) + 8 * hg) * (8 * K) + lane * K;
-        stream_block_rows<K, CB, 1, true>(base, row_words, blk * 8, blk * 8 + 8,
-                                          x + (size_t)(s / top_k) * D, (size_t)D, 1,
-                                          gu_suh + ((size_t)e * 2 + p) * D, xs[wave], lane, acc);
+        stream_block_rows<K, CB, 1, true, kHalf>(base, row_words, tk0, tk0 + (kHalf ? 4 : 8),
+                                                 x + (size_t)(s / top_k) * D, (size_t)D, 1,
+                                                 gu_suh + ((size_t)e * 2 + p) * D, xs[wave], lane,
+                                                 acc);
     }
-    const float2_t v = moe_wg_sum(red, acc, lane, wave);
+    const float2_t v = moe_wg_sum<NW>(red, acc, lane, wave);
     int* counter = counters + s * hblocks + hg;
     if (wave == 0) {
         const bool last = moe_publish(part + ((size_t)gid * n_wg + blockIdx.y) * 128, v, counter,
@@ -284,13 +294,13 @@ __global__ __launch_bounds__(256) void moe_gateup_kernel(
 
 // grid = (slots * D/128, ceil((H/128) / 4)); slot s = gid / dblocks, column block
 // og = gid % dblocks. xh_dn is already rotated. part: fp32 [gid][n_wg][128].
-template <int K, int CB>
-__global__ __launch_bounds__(256) void moe_down_kernel(
+template <int K, int CB, int NW>
+__global__ __launch_bounds__(NW * 64) void moe_down_kernel(
     const uint32_t* __restrict__ dn_trellis, const half_t* __restrict__ xh_dn,
     const int* __restrict__ indices, const half_t* __restrict__ dn_svh, half_t* __restrict__ y,
     float* part, int* counters, int E, int D, int H) {
-    __shared__ __attribute__((aligned(16))) half_t xs[4][1][kXwLd];
-    __shared__ float red[4][128];
+    __shared__ __attribute__((aligned(16))) half_t xs[NW][1][kXwLd];
+    __shared__ float red[NW][128];
     __shared__ int last_flag;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -299,16 +309,19 @@ __global__ __launch_bounds__(256) void moe_down_kernel(
     const int gid = blockIdx.x;
     const int og = gid % dblocks, s = gid / dblocks;
     const int e = clamp_expert(indices[s], E);
-    const int blk = blockIdx.y * 4 + wave;
+    constexpr bool kHalf = NW == 8;
+    const int part_idx = blockIdx.y * NW + wave;
+    const int blk = kHalf ? part_idx >> 1 : part_idx;
+    const int tk0 = blk * 8 + (kHalf ? (part_idx & 1) * 4 : 0);
     float acc[1][2] = {{0.f, 0.f}};
     if (blk < hblocks) {
         const size_t row_words = (size_t)E * (D >> 4) * (8 * K);
         const uint32_t* base = dn_trellis + ((size_t)e * (D >> 4) + 8 * og) * (8 * K) + lane * K;
-        stream_block_rows<K, CB, 1, false>(base, row_words, blk * 8, blk * 8 + 8,
-                                           xh_dn + (size_t)s * H, (size_t)H, 1, nullptr, xs[wave],
-                                           lane, acc);
+        stream_block_rows<K, CB, 1, false, kHalf>(base, row_words, tk0, tk0 + (kHalf ? 4 : 8),
+                                                  xh_dn + (size_t)s * H, (size_t)H, 1, nullptr,
+                                                  xs[wave], lane, acc);
     }
-    float2_t v = moe_wg_sum(red, acc, lane, wave);
+    float2_t v = moe_wg_sum<NW>(red, acc, lane, wave);
     if (n_wg > 1) {
         int* counter = counters + gid;
         if (wave == 0) {
@@ -340,6 +353,13 @@ struct MoeWorkspace {
     GemvPlan plan_gu, plan_dn;
     int g_gu, g_dn;
 };
+
+// Two-launch chain: below this many whole-block waves in the gate/up launch the waves
+// take half blocks (4096 = four per SIMD).
+static int moe_half_below() {
+    static const int v = env_int("EXL3_MOE_HALF_BELOW", 4096, 0, 1 << 20);
+    return v;
+}
 
 static MoeWorkspace moe_workspace(int tokens, int top_k, int D, int H) {
     MoeWorkspace w{};
@@ -546,22 +566,30 @@ EXL3_EXPORT int exl3_moe_forward(const uint16_t* x, int tokens, const int32_t* i
         // two launches: gate/up + GLU + rotation, then down
         const int hblocks = H / 128, dblocks = D / 128;
         if (counters_len < (size_t)slots * (hblocks + dblocks)) return EXL3_E_WORKSPACE;
-        return dispatch_k_cb(K, cb, [&](auto k, auto c) {
-            moe_gateup_kernel<k.value, c.value>
-                <<<dim3((unsigned)(slots * 2 * hblocks), (unsigned)((dblocks + 3) / 4)), dim3(256),
-                   0, s>>>(reinterpret_cast<const uint32_t*>(gu_trellis),
-                           reinterpret_cast<const half_t*>(x), indices,
-                           reinterpret_cast<const half_t*>(gu_suh),
-                           reinterpret_cast<const half_t*>(gu_svh),
-                           reinterpret_cast<const half_t*>(dn_suh), xh_dn, part_gu, counters,
-                           top_k, num_experts, D, H, activation);
+        // few slots: eight waves per workgroup, each on half a block, so that the
+        // chip holds twice the loads in flight (same workgroup count, same partial rows)
+        const bool half = (size_t)slots * 2 * hblocks * dblocks < (size_t)moe_half_below();
+        auto chain = [&](auto k, auto c, auto nw) {
+            constexpr int NW = nw.value;
+            moe_gateup_kernel<k.value, c.value, NW>
+                <<<dim3((unsigned)(slots * 2 * hblocks), (unsigned)((dblocks + 3) / 4)),
+                   dim3(NW * 64), 0, s>>>(reinterpret_cast<const uint32_t*>(gu_trellis),
+                                          reinterpret_cast<const half_t*>(x), indices,
+                                          reinterpret_cast<const half_t*>(gu_suh),
+                                          reinterpret_cast<const half_t*>(gu_svh),
+                                          reinterpret_cast<const half_t*>(dn_suh), xh_dn, part_gu,
+                                          counters, top_k, num_experts, D, H, activation);
             if (int rc = launch_status()) return rc;
-            moe_down_kernel<k.value, c.value>
-                <<<dim3((unsigned)(slots * dblocks), (unsigned)((hblocks + 3) / 4)), dim3(256), 0,
-                   s>>>(reinterpret_cast<const uint32_t*>(dn_trellis), xh_dn, indices,
-                        reinterpret_cast<const half_t*>(dn_svh), reinterpret_cast<half_t*>(y),
-                        part_dn, counters + (size_t)slots * hblocks, num_experts, D, H);
+            moe_down_kernel<k.value, c.value, NW>
+                <<<dim3((unsigned)(slots * dblocks), (unsigned)((hblocks + 3) / 4)), dim3(NW * 64),
+                   0, s>>>(reinterpret_cast<const uint32_t*>(dn_trellis), xh_dn, indices,
+                           reinterpret_cast<const half_t*>(dn_svh), reinterpret_cast<half_t*>(y),
+                           part_dn, counters + (size_t)slots * hblocks, num_experts, D, H);
             return launch_status();
+        };
+        return dispatch_k_cb(K, cb, [&](auto k, auto c) {
+            return half ? chain(k, c, std::integral_constant<int, 8>{})
+                        : chain(k, c, std::integral_constant<int, 4>{});
         });
     }
 
