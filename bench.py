@@ -16,7 +16,7 @@ Prints ONE JSON line: metric, value, unit, n_gpus, steps, warmup, ms_per_step,
 higher_is_better, scaling, vs_baseline, dtype, data, config, plus the objects
 roofline (dominant kernel = the one-launch layer kernel, launch durations from
 HIP events around batched graph replays on cold weights), cpu_baseline (the C
-oracle on the host cores), batch_rows (2/4/8 rows), config1, prefill_gemm
+oracle on the host cores), batch_rows (2..128 rows), config1, prefill_gemm
 (M=2048, config 3), moe (config 4) and, with --sweep, config5.
 """
 
@@ -364,7 +364,9 @@ def _launch_ms(lin, x, k, dev, cb=CB, min_bytes=320e6, reps=20):
     gen = torch.Generator(device=dev).manual_seed(31_000 + lin.n_in + lin.n_out + k)
     trs = [torch.randint(-32768, 32768, (lin.n_in // 16, lin.n_out // 16, 16 * k), dtype=torch.int16,
                          device=dev, generator=gen) for _ in range(copies)]
-    call = lambda tr: ops.linear_forward(x, tr, k, cb, lin.suh, lin.svh, None, lin.group_sub)
+    call = lambda tr: ops.linear_forward(x, tr, k, cb, lin.suh, lin.svh, None, lin.group_sub,
+                                         member_out=lin.outs if lin.members > 1 else None,
+                                         block_sub=lin.block_sub)
     for tr in trs:
         call(tr)
     torch.cuda.synchronize()
@@ -401,12 +403,13 @@ def _rows_x(n, rows, dev):
 
 
 def bench_batch_rows(dev, layer):
-    """The same layer step at 2, 4, 8 and 16 rows (batched decode, speculative verify):
-    sum of the launch durations on cold weights (at 16 rows each linear is the input
-    rotation launch plus the one-launch kernel)."""
+    """The same layer step at 2 .. 128 rows (batched decode, speculative verify):
+    sum of the launch durations on cold weights (9..32 rows: each linear is the
+    input rotation launch plus the medium-batch kernel; above that the rotation, the
+    prefill GEMM with every tile split and its fix-up pass)."""
     res = {}
     total = sum(l.bytes for l in layer)
-    for rows in (2, 4, 8, 16):
+    for rows in (2, 4, 8, 16, 32, 64, 128):
         ms = sum(_launch_ms(lin, _rows_x(lin.n_in, rows, dev), K_BITS, dev) for lin in layer)
         res[f"rows_{rows}"] = {"us_per_step": round(ms * 1e3, 2), "GBps": round(total / ms / 1e6, 1)}
     return {"batch_rows": res}

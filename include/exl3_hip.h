@@ -49,9 +49,10 @@ const char *exl3_status_string(int status);
 /* Largest row count the small-batch kernel (exl3_gemv) accepts per call. */
 int exl3_gemv_max_rows(void);
 
-/* Largest row count exl3_linear_forward serves with its one-launch small-batch
- * kernel when given counters (above exl3_gemv_max_rows() the input rotation runs
- * as a launch of its own first). Beyond it the prefill GEMM takes over. */
+/* Largest row count exl3_linear_forward serves with its small- and medium-batch
+ * kernels when given counters (stacked suh included; above exl3_gemv_max_rows()
+ * the input rotation runs as a launch of its own first). Beyond it the prefill
+ * GEMM takes over. */
 int exl3_linear_small_max_rows(void);
 
 /*
@@ -228,8 +229,11 @@ size_t exl3_gemm_workspace_bytes(int rows, int in_tiles, int tn_count);
  *            and applies the output transform. The array must be all zero on
  *            entry and is all zero again when the launch has finished, so a
  *            caller zeroes it once and reuses it (calls that overlap on one
- *            array race). NULL selects the three-launch chain
- *            (exl3_had128_pre, exl3_gemv_partials, exl3_had128_post).
+ *            array race). Above that and up to exl3_linear_small_max_rows() rows
+ *            the counters serve the medium-batch kernel in the same way (two
+ *            launches: input rotation, then everything else). NULL selects the
+ *            three-launch chain (exl3_had128_pre, exl3_gemv_partials,
+ *            exl3_had128_post) resp. the prefill GEMM.
  */
 int exl3_linear_forward(const uint16_t *x, int rows, const uint16_t *trellis, int in_tiles,
                         int out_tiles, int K, int cb, const uint16_t *suh, int n_sub,

@@ -9,7 +9,7 @@ namespace exl3 {
 //   [0, xh_bytes)            xh  fp16 [rows][n_sub][in]
 //   [xh_bytes, ...)          rows <= kGemvMaxRows: fp32 split-K partials
 //                            otherwise:            fp16 y [rows][out], or (rows <=
-//                            kLinearSmallMaxRows, one-launch kernel) fp32 partials
+//                            kLinearMidMaxRows, medium-batch kernel) fp32 partials
 //   then (rows > kGemvMaxRows) the fp32 partial tiles of the prefill GEMM
 struct LinearWorkspace {
     size_t xh_bytes;
@@ -28,10 +28,10 @@ static LinearWorkspace linear_workspace(int rows, int in_features, int out_featu
         w.second_bytes = (size_t)n * rows * out_features * sizeof(float);
     } else {
         w.second_bytes = (size_t)rows * out_features * 2;
-        if (rows <= kLinearSmallMaxRows) {
-            const GemvPlan b = plan_linear_small(rows, in_features / 16, out_features / 128);
-            const size_t small = (size_t)b.n_partials() * rows * out_features * sizeof(float);
-            if (small > w.second_bytes) w.second_bytes = small;
+        if (rows <= kLinearMidMaxRows) {
+            const MidPlan m = plan_linear_mid(rows, in_features / 16, out_features / 128);
+            const size_t mid = (size_t)m.n_splits * rows * out_features * sizeof(float);
+            if (mid > w.second_bytes) w.second_bytes = mid;
         }
         w.gemm_bytes = align_up(gemm_workspace_bytes(rows, in_features / 16, out_features / 16), 256);
     }
@@ -92,7 +92,7 @@ EXL3_EXPORT int exl3_linear_forward(const uint16_t* x, int rows, const uint16_t*
             if (counters_len < (size_t)n_groups) return EXL3_E_WORKSPACE;
             return launch_linear_small(x, rows, trellis, in_tiles, out_tiles, K, cb, suh, n_sub,
                                        group_sub, svh, bias, y, partial, counters,
-                                       plan_linear_small(rows, in_tiles, n_groups), false, s);
+                                       plan_linear_small(rows, in_tiles, n_groups), s);
         }
         if (int rc = launch_had_pre(x, rows, in_features, suh, n_sub, xh, s)) return rc;
         if (int rc = launch_gemv_partials(xh, rows, n_sub, trellis, in_tiles, out_tiles, K, cb,
@@ -104,15 +104,15 @@ EXL3_EXPORT int exl3_linear_forward(const uint16_t* x, int rows, const uint16_t*
 
     // Prefill: rotation kernel, MFMA GEMM, output transform.
     if (int rc = launch_had_pre(x, rows, in_features, suh, n_sub, xh, s)) return rc;
-    if (rows <= kLinearSmallMaxRows && counters) {
-        // 9..16 rows: the decode sets the pace, not the matrix cores; the small-batch
-        // kernel (every weight decoded once, dot products on 4x4x4 MFMA) on the
-        // rotated rows, split reduction and output transform in the same launch
+    if (counters && rows <= linear_mid_max_rows()) {
+        // a few dozen rows: the decode still sets the pace; every weight is decoded
+        // once and goes from registers into 16x16x32 MFMA; split reduction and output
+        // transform in the same launch
         const int n_groups = out_tiles / 8;
         if (counters_len < (size_t)n_groups) return EXL3_E_WORKSPACE;
-        return launch_linear_small(xh, rows, trellis, in_tiles, out_tiles, K, cb, nullptr, n_sub,
-                                   group_sub, svh, bias, y, reinterpret_cast<float*>(second),
-                                   counters, plan_linear_small(rows, in_tiles, n_groups), true, s);
+        return launch_linear_mid(xh, rows, trellis, in_tiles, out_tiles, K, cb, n_sub, group_sub,
+                                 svh, bias, y, reinterpret_cast<float*>(second), counters,
+                                 plan_linear_mid(rows, in_tiles, n_groups), s);
     }
     uint16_t* ytmp = reinterpret_cast<uint16_t*>(second);
     if (n_sub == 1) {

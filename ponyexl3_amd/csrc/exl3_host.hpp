@@ -69,15 +69,30 @@ int launch_gemv_partials(const uint16_t* xh, int rows, int n_sub, const uint16_t
                          hipStream_t stream);
 
 // One-launch small-batch layer (rows <= kLinearSmallMaxRows): counters[out_tiles/8]
-// must be zero on entry and are zero again on exit. Up to kGemvMaxRows rows the
-// kernel rotates x itself (pre_rotated = false); above that x must be the output
-// of launch_had_pre, fp16 [rows][n_sub][in] (pre_rotated = true, suh not applied).
-constexpr int kLinearSmallMaxRows = 16;
+// must be zero on entry and are zero again on exit. The kernel rotates x itself.
+constexpr int kLinearSmallMaxRows = kGemvMaxRows;
 int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, int in_tiles,
                         int out_tiles, int K, int cb, const uint16_t* suh, int n_sub,
                         const int32_t* group_sub, const uint16_t* svh, const uint16_t* bias,
                         uint16_t* y, float* partial, int* counters, GemvPlan plan,
-                        bool pre_rotated, hipStream_t stream);
+                        hipStream_t stream);
+
+// Medium-batch layer (rows <= kLinearMidMaxRows) on rotated activations xh, fp16
+// [rows][n_sub][in]: weights decoded once and fed to 16x16x16 MFMA from registers;
+// partial: fp32 [plan.n_splits][rows][out]; counters as for launch_linear_small.
+constexpr int kLinearMidMaxRows = 32;
+struct MidPlan {
+    int n_splits;          // workgroups per 128-column group
+    int blocks_per_split;  // 128-row blocks of the reduction per workgroup
+};
+MidPlan plan_linear_mid(int rows, int in_tiles, int n_groups);
+// Largest row count that exl3_linear_forward sends to it (it starts above
+// kLinearSmallMaxRows; a value below that switches it off).
+int linear_mid_max_rows();
+int launch_linear_mid(const uint16_t* xh, int rows, const uint16_t* trellis, int in_tiles,
+                      int out_tiles, int K, int cb, int n_sub, const int32_t* group_sub,
+                      const uint16_t* svh, const uint16_t* bias, uint16_t* y, float* partial,
+                      int* counters, MidPlan plan, hipStream_t stream);
 
 int launch_had_pre(const uint16_t* x, int rows, int n, const uint16_t* suh, int n_sub,
                    uint16_t* xh, hipStream_t stream);

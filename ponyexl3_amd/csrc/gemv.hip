@@ -185,18 +185,14 @@ __global__ __launch_bounds__(256) void gemv_kernel(
 //     deterministic.
 // Counters must be zero on entry; they are zero again when the kernel ends.
 //
-// ROTATE = false (9..16 rows): x is already rotated, fp16 [rows][n_sub][in], one
-// input transform per sibling done by the Hadamard kernel; the waves only stage
-// it. Rotating sixteen rows in every workgroup would cost more instructions than
-// the decode itself.
 // HALF (one and two rows only): splits are half blocks of four tile rows.
-template <int K, int CB, int MT, bool ROTATE, bool HALF>
+template <int K, int CB, int MT, bool HALF>
 __global__ __launch_bounds__(256) void linear_small_kernel(
     const uint32_t* __restrict__ trellis, const half_t* __restrict__ x,
     const half_t* __restrict__ suh, const half_t* __restrict__ svh,
     const half_t* __restrict__ bias, half_t* __restrict__ y, float* partial, int* counters,
     const int* __restrict__ group_sub, int in_tiles, int out_tiles, int rows, int n_groups,
-    int tk_per_split, int n_splits, int n_sub) {
+    int tk_per_split, int n_splits) {
     __shared__ __attribute__((aligned(16))) half_t xs[4][MT][kXwLd];
     const int g = blockIdx.x;
     const int lane = threadIdx.x & 63;
@@ -209,9 +205,7 @@ __global__ __launch_bounds__(256) void linear_small_kernel(
     const int tk_end = active ? min(in_tiles, tk_begin + tk_per_split) : 0;
     const size_t row_words = (size_t)out_tiles * (8 * K);
     const uint32_t* base = trellis + (size_t)g * 8 * (8 * K) + lane * K;
-    const half_t* suh_row = ROTATE && suh ? suh + (size_t)sub * in_features : nullptr;
-    const half_t* x_rows = ROTATE ? x : x + (size_t)sub * in_features;
-    const size_t x_stride = ROTATE ? (size_t)in_features : (size_t)n_sub * in_features;
+    const half_t* suh_row = suh ? suh + (size_t)sub * in_features : nullptr;
 
     float acc[MT][2];
 #pragma unroll
@@ -219,8 +213,9 @@ __global__ __launch_bounds__(256) void linear_small_kernel(
 
     // ---- input Hadamard (or staging) + decode/dot pipeline over this wave's blocks
     if (active)
-        stream_block_rows<K, CB, MT, ROTATE, HALF>(base, row_words, tk_begin, tk_end, x_rows,
-                                                   x_stride, rows, suh_row, xs[wave], lane, acc);
+        stream_block_rows<K, CB, MT, true, HALF>(base, row_words, tk_begin, tk_end, x,
+                                                 (size_t)in_features, rows, suh_row, xs[wave], lane,
+                                                 acc);
 
     // ---- the four waves of the workgroup are summed through LDS in wave order,
     // the workgroup stores ONE fp32 partial row, and the last workgroup of the
@@ -411,16 +406,13 @@ int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, in
                         int out_tiles, int K, int cb, const uint16_t* suh, int n_sub,
                         const int32_t* group_sub, const uint16_t* svh, const uint16_t* bias,
                         uint16_t* y, float* partial, int* counters, GemvPlan plan,
-                        bool pre_rotated, hipStream_t stream) {
+                        hipStream_t stream) {
     if (int rc = check_k_cb(K, cb)) return rc;
     if (!x || !trellis || !y || !partial || !counters) return EXL3_E_NULL_POINTER;
     if (rows < 1 || rows > kLinearSmallMaxRows || n_sub < 1 || in_tiles < 8 || out_tiles < 8 ||
         in_tiles % 8 || out_tiles % 8)
         return EXL3_E_BAD_SHAPE;
-    // the in-kernel rotation exists for up to kGemvMaxRows rows, the staging-only
-    // variant for the row counts above that
-    if (pre_rotated != (rows > kGemvMaxRows)) return EXL3_E_UNSUPPORTED;
-    if (n_sub > 1 && (!group_sub || (!suh && !pre_rotated))) return EXL3_E_BAD_INDEX;
+    if (n_sub > 1 && (!group_sub || !suh)) return EXL3_E_BAD_INDEX;
     const bool half = plan.tk_per_split == 4 && rows <= 2;
     if (plan.n_splits < 1 || plan.n_splits > 4 * 65535 ||
         (!half && (plan.tk_per_split < 8 || plan.tk_per_split % 8)) ||
@@ -428,31 +420,30 @@ int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, in
         return EXL3_E_BAD_SHAPE;
     const int n_groups = out_tiles / 8;
     const dim3 grid((unsigned)n_groups, (unsigned)((plan.n_splits + 3) / 4));
-    const int mt = rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : rows <= 8 ? 8 : 16;
+    const int mt = rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8;
     return dispatch_k_cb(K, cb, [&](auto k, auto c) {
-        auto go = [&](auto mtc, auto rot, auto halfc) {
-            linear_small_kernel<k.value, c.value, mtc.value, rot.value, halfc.value>
+        auto go = [&](auto mtc, auto halfc) {
+            linear_small_kernel<k.value, c.value, mtc.value, halfc.value>
                 <<<grid, dim3(256), 0, stream>>>(
                     reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<const half_t*>(x),
                     reinterpret_cast<const half_t*>(suh), reinterpret_cast<const half_t*>(svh),
                     reinterpret_cast<const half_t*>(bias), reinterpret_cast<half_t*>(y), partial,
                     counters, group_sub, in_tiles, out_tiles, rows, n_groups, plan.tk_per_split,
-                    plan.n_splits, n_sub);
+                    plan.n_splits);
         };
         using T = std::true_type;
         using F = std::false_type;
         switch (mt) {
             case 1:
-                if (half) go(std::integral_constant<int, 1>{}, T{}, T{});
-                else go(std::integral_constant<int, 1>{}, T{}, F{});
+                if (half) go(std::integral_constant<int, 1>{}, T{});
+                else go(std::integral_constant<int, 1>{}, F{});
                 break;
             case 2:
-                if (half) go(std::integral_constant<int, 2>{}, T{}, T{});
-                else go(std::integral_constant<int, 2>{}, T{}, F{});
+                if (half) go(std::integral_constant<int, 2>{}, T{});
+                else go(std::integral_constant<int, 2>{}, F{});
                 break;
-            case 4: go(std::integral_constant<int, 4>{}, T{}, F{}); break;
-            case 8: go(std::integral_constant<int, 8>{}, T{}, F{}); break;
-            default: go(std::integral_constant<int, 16>{}, F{}, F{}); break;
+            case 4: go(std::integral_constant<int, 4>{}, F{}); break;
+            default: go(std::integral_constant<int, 8>{}, F{}); break;
         }
         return launch_status();
     });
@@ -462,7 +453,11 @@ int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, in
 
 EXL3_EXPORT int exl3_gemv_max_rows(void) { return exl3::kGemvMaxRows; }
 
-EXL3_EXPORT int exl3_linear_small_max_rows(void) { return exl3::kLinearSmallMaxRows; }
+EXL3_EXPORT int exl3_linear_small_max_rows(void) {
+    // the medium-batch kernel continues where the small-batch one ends
+    const int mid = exl3::linear_mid_max_rows();
+    return mid > exl3::kLinearSmallMaxRows ? mid : exl3::kLinearSmallMaxRows;
+}
 
 EXL3_EXPORT size_t exl3_gemv_workspace_bytes(int rows, int in_tiles, int n_groups) {
     if (rows < 1 || in_tiles < 1 || n_groups < 1) return 0;

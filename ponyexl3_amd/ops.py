@@ -286,7 +286,8 @@ def gemv_max_rows() -> int:
 
 
 def linear_small_max_rows() -> int:
-    """Rows up to which ``linear_forward(fused=True)`` uses the one-launch kernel."""
+    """Rows up to which ``linear_forward(fused=True)`` uses the small- and
+    medium-batch kernels (stacked ``suh`` included); above it the prefill GEMM runs."""
     return int(_lib.load().exl3_linear_small_max_rows())
 
 

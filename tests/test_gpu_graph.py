@@ -36,7 +36,7 @@ def _replay_matches_eager(cuda, make_inputs, run, n_replays=4):
 @pytest.mark.parametrize("rows", [1, 4, 8, 12, 40])
 def test_layer_step_replays(cuda, rows):
     """One decoder layer's linears (sibling-fused qkv-like group, a plain layer with
-    bias) at small-batch, 9..16-row and prefill row counts."""
+    bias) at small-batch, medium-batch (9..32 rows) and prefill row counts."""
     from ponyexl3_amd import EXL3Linear, FusedEXL3Group, make_exl3_layer
 
     group = FusedEXL3Group([make_exl3_layer(k=4, in_features=512, out_features=o, seed=40 + i, key=f"g{i}")

@@ -61,8 +61,9 @@ def test_module_matches_oracle(cuda, oracle, rows, k, mcg):
 @pytest.mark.parametrize("cb", [0, 1, 2])
 def test_every_k_codebook_and_row_count(cuda, oracle, k, cb):
     """Every bit width, codebook and small-batch row count (each row count up to 8
-    is its own instruction schedule in the one-launch kernel), both launch plans,
-    plus two prefill row counts, against the oracle."""
+    is its own instruction schedule in the one-launch kernel), row counts of the
+    medium-batch kernel (9..32 rows; 70 rows are prefill), both launch
+    plans, against the oracle."""
     from ponyexl3_amd import make_exl3_layer, ops
 
     layer = make_exl3_layer(k=k, in_features=256, out_features=256, seed=300 + 10 * k + cb,
@@ -71,15 +72,15 @@ def test_every_k_codebook_and_row_count(cuda, oracle, k, cb):
     suh, svh = torch.from_numpy(layer.suh).to(cuda), torch.from_numpy(layer.svh).to(cuda)
     bias = torch.from_numpy(layer.bias).to(cuda)
     rng = np.random.default_rng(k * 3 + cb)
-    for rows in (1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 16, 17, 70):
+    for rows in (1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 16, 17, 31, 70):
         x, xt = _x(rng, (rows, 256), cuda)
         ref = _oracle_forward(oracle, layer, x)
         print(f"k={k} cb={cb} rows={rows}", flush=True)
         y = ops.linear_forward(xt, tr, k, cb, suh, svh, bias, fused=True).cpu().numpy()
         assert rel_l2(y, ref) <= TOL, f"one-launch rows={rows}"
-        if rows <= 16:  # the launch chain (up to 8 rows) / the prefill GEMM (9..16)
-            y = ops.linear_forward(xt, tr, k, cb, suh, svh, bias, fused=False).cpu().numpy()
-            assert rel_l2(y, ref) <= TOL, f"chain rows={rows}"
+        # the launch chain (up to 8 rows) / the prefill GEMM (from 9 rows on)
+        y = ops.linear_forward(xt, tr, k, cb, suh, svh, bias, fused=False).cpu().numpy()
+        assert rel_l2(y, ref) <= TOL, f"chain rows={rows}"
 
 
 def test_general_scales_not_only_signs(cuda, oracle):
@@ -196,8 +197,8 @@ def test_single_slot_cache_computes_once(cuda):
 @pytest.mark.parametrize("k,n_in,n_out", [(4, 512, 384), (3, 1024, 256), (6, 2176, 640), (4, 5120, 1024)])
 def test_one_launch_layer_equals_three_launch_chain(cuda, rows, k, n_in, n_out):
     """The fused kernel (rotation + GEMV + last-wave reduction + output transform;
-    from 9 rows on with the rotation as its own launch) against the chained
-    kernels (from 9 rows on the prefill GEMM). Both add the same fp32 products, but cut the
+    from 9 rows on the medium-batch kernel behind a rotation launch) against the
+    chained kernels (from 9 rows on the prefill GEMM). Both add the same fp32 products, but cut the
     reduction dimension at different tile rows, so the sums can differ in the last
     fp32 bit and, rarely, flip an fp16 rounding before the output Hadamard: they
     must agree to a few fp16 ulps of the largest output. The fused kernel must be
@@ -220,6 +221,55 @@ def test_one_launch_layer_equals_three_launch_chain(cuda, rows, k, n_in, n_out):
         diff = float((a.float() - b.float()).abs().max())
         assert diff <= 2e-3 * float(b.float().abs().max()), f"rep {rep}: {diff}"
     assert int(ops.sync_counters(cuda, 1).abs().sum()) == 0
+
+
+@pytest.mark.parametrize("rows", [9, 13, 16, 17, 25, 32])
+@pytest.mark.parametrize("k,cb,n_in,n_out", [(4, 0, 2176, 640), (3, 1, 4096, 384), (5, 0, 1024, 1280),
+                                             (8, 2, 1152, 256), (7, 0, 640, 128), (6, 1, 2048, 256),
+                                             (2, 0, 1536, 384), (1, 0, 1024, 256)])
+def test_medium_batch_kernel(cuda, oracle, rows, k, cb, n_in, n_out):
+    """9..32 rows with counters: rotation launch, then the kernel whose lanes own the
+    tensor-core fragments of the trellis format and feed them to 16x16x32 MFMA from
+    registers; the reduction is cut into splits of unequal length that meet through
+    partial rows and the group counters. Against the oracle, against
+    the prefill GEMM on the same input (same fp32 products, other cut points), and
+    bit-identical twice in a row with the counters back at zero."""
+    from ponyexl3_amd import make_exl3_layer, ops
+
+    assert ops.linear_small_max_rows() >= 32
+    layer = make_exl3_layer(k=k, in_features=n_in, out_features=n_out, seed=40 * k + cb + rows,
+                            mcg=cb == 1, mul1=cb == 2, bias=True)
+    tr = ops.as_trellis_tensor(layer.trellis, cuda)
+    suh, svh = torch.from_numpy(layer.suh).to(cuda), torch.from_numpy(layer.svh).to(cuda)
+    bias = torch.from_numpy(layer.bias).to(cuda)
+    rng = np.random.default_rng(rows + k)
+    x, xt = _x(rng, (rows, n_in), cuda)
+    print(f"medium batch rows={rows} k={k} cb={cb} {n_in}->{n_out}", flush=True)
+    a = ops.linear_forward(xt, tr, k, cb, suh, svh, bias, fused=True)
+    a2 = ops.linear_forward(xt, tr, k, cb, suh, svh, bias, fused=True)
+    assert torch.equal(a, a2)
+    assert int(ops.sync_counters(cuda, 1).abs().sum()) == 0
+    assert rel_l2(a.cpu().numpy(), _oracle_forward(oracle, layer, x)) <= TOL
+    b = ops.linear_forward(xt, tr, k, cb, suh, svh, bias, fused=False)
+    diff = float((a.float() - b.float()).abs().max())
+    assert diff <= 2e-3 * float(b.float().abs().max())
+
+
+@pytest.mark.parametrize("rows", [12, 20, 32])
+def test_medium_batch_kernel_sibling_group(cuda, oracle, rows):
+    """Stacked siblings (each 128-column group reads its member's rotation) through
+    the medium-batch kernel, members of 384, 256 and 128 columns."""
+    from ponyexl3_amd import FusedEXL3Group, make_exl3_layer
+
+    layers = [make_exl3_layer(k=4, in_features=1280, out_features=o, seed=270 + i, key=f"m{i}")
+              for i, o in enumerate((384, 256, 128))]
+    group = FusedEXL3Group(layers)
+    rng = np.random.default_rng(rows)
+    x, xt = _x(rng, (rows, 1280), cuda)
+    print(f"medium batch siblings rows={rows}", flush=True)
+    for o, l in zip(group.forward_all(xt), layers):
+        assert tuple(o.shape) == (rows, l.out_features)
+        assert rel_l2(o.cpu().numpy(), _oracle_forward(oracle, l, x)) <= TOL
 
 
 @pytest.mark.parametrize("rows", [17, 33, 64, 100, 130])
@@ -260,9 +310,17 @@ def test_sibling_prefill_in_one_gemm_launch(cuda, oracle, rows):
     x, xt = _x(rng, (rows, 1024), cuda)
     print(f"sibling prefill rows={rows}", flush=True)
     outs = group.forward_all(xt)
+    # fused=False keeps the prefill GEMM also at row counts that the medium-batch
+    # kernel would otherwise take
+    y_gemm = ops.linear_forward(xt, group._trellis, group._k, group._cb, group._suh_stack, group._svh_cat,
+                                None, group._group_sub, fused=False, member_out=group._out_features,
+                                block_sub=group._block_sub)
+    outs_gemm = torch.split(y_gemm, group._out_features, dim=-1)
     xh = ops.had128_pre(xt, group._suh_stack)
     for i, (o, l) in enumerate(zip(outs, layers)):
         assert rel_l2(o.cpu().numpy(), _oracle_forward(oracle, l, x)) <= TOL
+        assert rel_l2(outs_gemm[i].cpu().numpy(), _oracle_forward(oracle, l, x)) <= TOL
+        o = outs_gemm[i]
         member = ops.had128_post(ops.inner_gemm(xh[:, i].contiguous(), ops.as_trellis_tensor(l.trellis, cuda),
                                                 4, int(l.codebook_mode)),
                                  torch.from_numpy(l.svh).to(cuda))

@@ -45,12 +45,14 @@ def test_moe_matches_oracle(cuda, oracle, tokens, k, mcg, act):
     assert rel_l2(y[0], ref) <= TOL
 
 
-@pytest.mark.parametrize("tokens", [1, 8])
+@pytest.mark.parametrize("tokens", [1, 8, 48])
 def test_two_launch_and_five_launch_chains(cuda, oracle, tokens):
     """D and H of five Hadamard blocks each: both kernels of the two-launch chain
     run two workgroups per column block (one of them with a single active wave)
-    and meet through the counters. Checked against the oracle, against the
-    five-launch chain, and twice in a row (the counters must be left at zero)."""
+    and meet through the counters. 1 and 8 tokens take the eight-wave workgroups
+    on half blocks, 48 tokens (96 slots) the four-wave ones on whole blocks.
+    Checked against the oracle, against the five-launch chain, and twice in a row
+    (the counters must be left at zero)."""
     from ponyexl3_amd import EXL3SwitchGLU, ops
 
     E, D, H, kk, k = 5, 640, 640, 2, 4
@@ -67,6 +69,7 @@ def test_two_launch_and_five_launch_chains(cuda, oracle, tokens):
     y2 = ops.moe_forward(*args, fused=True)
     y5 = ops.moe_forward(*args, fused=False)
     assert torch.equal(y1, y2)
+    assert int(ops.sync_counters(cuda, 1).abs().sum()) == 0
     ref = _oracle_chain(oracle, gate, up, down, x, idx, "silu")
     assert rel_l2(y1.cpu().numpy(), ref) <= TOL
     assert rel_l2(y5.cpu().numpy(), ref) <= TOL
