@@ -103,10 +103,16 @@ __global__ __launch_bounds__(256, 2) void linear_mid_kernel(
     constexpr int NL = (16 * K + 63) / 64;  // wave-wide loads that cover one tile pair
     constexpr int kDepth = 2;  // blocks ahead that a wave has its loads out for
     // Activations of one 128-row block, two buffers, laid out as the A operands of
-    // the matrix instruction: [fragment][row pair of the block][lane][8 halfs].
-    // After the main loop the same memory holds the fp32 sums of the workgroup.
-    __shared__ __attribute__((aligned(16))) half_t xs[2][MF][4][64][8];
-    static_assert(sizeof(xs) == (size_t)M * 128 * sizeof(float), "the sums reuse the staging memory");
+    // the matrix instruction: [buffer][fragment][row pair of the block][lane][8 halfs].
+    // After the main loop the same memory holds the fp32 sums of the workgroup: two
+    // [M][kRedLd] arrays (waves 0+1 and waves 2+3). kRedLd = 130 puts the four row
+    // groups of a lane quartet eight banks apart, so a wave's accesses are two per
+    // bank, the minimum for 64 lanes.
+    constexpr int kRedLd = 130;
+    constexpr size_t kStageBytes = (size_t)2 * MF * 4 * 64 * 8 * sizeof(half_t);
+    constexpr size_t kRedBytes = (size_t)2 * M * kRedLd * sizeof(float);
+    __shared__ __attribute__((aligned(16))) char lds_raw[kStageBytes > kRedBytes ? kStageBytes : kRedBytes];
+    half_t(*xs)[MF][4][64][8] = reinterpret_cast<half_t(*)[MF][4][64][8]>(lds_raw);
     __shared__ int last_flag;
     const int g = blockIdx.x;
     const int split = blockIdx.y;
@@ -264,12 +270,13 @@ __global__ __launch_bounds__(256, 2) void linear_mid_kernel(
         }
     }
 
-    // ---- the four waves' sums are added through LDS in wave order (the staging
-    // memory is free: the loop ended with a barrier)
-    float(*red)[128] = reinterpret_cast<float(*)[128]>(&xs[0][0][0][0][0]);
+    // ---- the four waves' sums are added through LDS, (wave 0 + wave 1) +
+    // (wave 2 + wave 3) (the staging memory is free: the loop ended with a barrier)
+    float(*red)[M][kRedLd] = reinterpret_cast<float(*)[M][kRedLd]>(lds_raw);
 #pragma unroll
-    for (int w = 0; w < 4; w++) {
-        if (wave == w) {
+    for (int phase = 0; phase < 2; phase++) {
+        if ((wave & 1) == phase) {
+            float(*dstbuf)[kRedLd] = red[wave >> 1];
 #pragma unroll
             for (int q = 0; q < 4; q++)
 #pragma unroll
@@ -278,9 +285,9 @@ __global__ __launch_bounds__(256, 2) void linear_mid_kernel(
                     for (int f = 0; f < MF; f++)
 #pragma unroll
                         for (int r = 0; r < 4; r++) {
-                            float* dst = &red[16 * f + 4 * kgroup + r]
-                                             [(2 * q + (col16 >> 3)) * 16 + (col16 & 7) + 8 * v];
-                            *dst = w == 0 ? acc[q][v][f][r] : __fadd_rn(*dst, acc[q][v][f][r]);
+                            float* dst = &dstbuf[16 * f + 4 * kgroup + r]
+                                                [(2 * q + (col16 >> 3)) * 16 + (col16 & 7) + 8 * v];
+                            *dst = phase == 0 ? acc[q][v][f][r] : __fadd_rn(*dst, acc[q][v][f][r]);
                         }
         }
         __syncthreads();
@@ -291,7 +298,8 @@ __global__ __launch_bounds__(256, 2) void linear_mid_kernel(
     const size_t out_total = (size_t)n_groups * 128;
     for (int idx = threadIdx.x; idx < rows * 64; idx += 256) {
         const int m = idx >> 6, c2 = idx & 63;
-        const float2_t v = {red[m][2 * c2], red[m][2 * c2 + 1]};
+        const float2_t v = {__fadd_rn(red[0][m][2 * c2], red[1][m][2 * c2]),
+                            __fadd_rn(red[0][m][2 * c2 + 1], red[1][m][2 * c2 + 1])};
         __hip_atomic_store(reinterpret_cast<uint64_t*>(partial + ((size_t)split * rows + m) * out_total +
                                                        (size_t)g * 128 + 2 * c2),
                            __builtin_bit_cast(uint64_t, v), __ATOMIC_RELAXED,
