@@ -188,32 +188,31 @@ __global__ __launch_bounds__(256, 2) void linear_mid_kernel(
         hi1 = half2_to_bits(w11);
     };
 
-    // staging of the activations: 16-byte chunks of a row, MF per thread and block;
-    // the four dwords of a chunk (input rows 2j, 2j+1 of one half of a tile row) go
-    // to the four k-groups' operands
+    // staging of the activations: 16-byte chunks of a row (input rows 2j, 2j+1 of one
+    // half of a tile row), MF per thread and block; the four dwords of a chunk go
+    // to the four k-groups' operands. Wave w stages row pair w: lane -> batch row
+    // lane >> 2 of a fragment, chunk lane & 3 of the pair, which spreads a store
+    // instruction over all LDS banks (two lanes per bank).
     const half_t* x_rows = xh + (size_t)sub * in_features;
     const size_t x_stride = (size_t)n_sub * in_features;
     uint4_t xr[MF];
     auto fetch_x = [&](int blk) {
 #pragma unroll
-        for (int i = 0; i < MF; i++) {
-            const int q = threadIdx.x + 256 * i;
-            const int r = min(q >> 4, rows - 1);
-            xr[i] = *reinterpret_cast<const uint4_t*>(x_rows + (size_t)r * x_stride + blk * 128 +
-                                                      (q & 15) * 8);
+        for (int f = 0; f < MF; f++) {
+            const int r = min(16 * f + (lane >> 2), rows - 1);
+            xr[f] = *reinterpret_cast<const uint4_t*>(x_rows + (size_t)r * x_stride + blk * 128 +
+                                                      (4 * wave + (lane & 3)) * 8);
         }
     };
     auto stage_x = [&](int which) {
+        const int odd = (lane >> 1) & 1, hi = lane & 1;  // tile row 2w + odd, upper half hi
 #pragma unroll
-        for (int i = 0; i < MF; i++) {
-            const int q = threadIdx.x + 256 * i;
-            const int m = q >> 4, c = q & 15;  // chunk c: tile row c >> 1, upper half c & 1
-            const int p = c >> 2, odd = (c >> 1) & 1, hi = c & 1;
-            const uint32_t d[4] = {xr[i].x, xr[i].y, xr[i].z, xr[i].w};
+        for (int f = 0; f < MF; f++) {
+            const uint32_t d[4] = {xr[f].x, xr[f].y, xr[f].z, xr[f].w};
 #pragma unroll
             for (int kg = 0; kg < 4; kg++)
                 *reinterpret_cast<uint32_t*>(
-                    &xs[which][m >> 4][p][16 * kg + (m & 15)][odd * 4 + hi * 2]) = d[kg];
+                    &xs[which][f][wave][16 * kg + (lane >> 2)][odd * 4 + hi * 2]) = d[kg];
         }
     };
 
