@@ -226,7 +226,7 @@ def test_one_launch_layer_equals_three_launch_chain(cuda, rows, k, n_in, n_out):
 @pytest.mark.parametrize("rows", [9, 13, 16, 17, 25, 32])
 @pytest.mark.parametrize("k,cb,n_in,n_out", [(4, 0, 2176, 640), (3, 1, 4096, 384), (5, 0, 1024, 1280),
                                              (8, 2, 1152, 256), (7, 0, 640, 128), (6, 1, 2048, 256),
-                                             (2, 0, 1536, 384), (1, 0, 1024, 256)])
+                                             (2, 0, 1536, 384), (1, 0, 1024, 256), (4, 1, 128, 128)])
 def test_medium_batch_kernel(cuda, oracle, rows, k, cb, n_in, n_out):
     """9..32 rows with counters: rotation launch, then the kernel whose lanes own the
     tensor-core fragments of the trellis format and feed them to 16x16x32 MFMA from
