@@ -230,7 +230,10 @@ __global__ __launch_bounds__(256, 2) void linear_mid_kernel(
     fetch_x(blk_begin);
     stage_x(0);
     if (blk_begin + 1 < blk_end) fetch_x(blk_begin + 1);
-    __syncthreads();
+    // a wave stages exactly the operands it reads itself (row pair w), so the
+    // waves of the workgroup never wait for each other inside the loop
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
 
     static_assert(kDepth % 2 == 0, "the staging buffer of a block is its ring slot & 1");
     for (int blk4 = blk_begin; blk4 < blk_end; blk4 += kDepth) {
@@ -265,12 +268,15 @@ __global__ __launch_bounds__(256, 2) void linear_mid_kernel(
                 }
             }
             load_pairs(blk + kDepth, ring[h]);
-            __syncthreads();  // this block's operands are consumed, the next block's are staged
+            // this block's operands are consumed, the next block's are staged
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
         }
     }
 
     // ---- the four waves' sums are added through LDS, (wave 0 + wave 1) +
-    // (wave 2 + wave 3) (the staging memory is free: the loop ended with a barrier)
+    // (wave 2 + wave 3), in the staging memory once every wave has left the loop
+    __syncthreads();
     float(*red)[M][kRedLd] = reinterpret_cast<float(*)[M][kRedLd]>(lds_raw);
 #pragma unroll
     for (int phase = 0; phase < 2; phase++) {
