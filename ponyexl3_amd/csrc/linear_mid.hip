@@ -23,10 +23,11 @@
 // Workgroup = one 128-column group (one block of the output Hadamard) over the
 // 128-row blocks of one split. Wave w takes tile rows 2w and 2w + 1 of every
 // block, on all four tile pairs, so that one activation operand serves eight
-// matrix instructions. The waves' sums are added through LDS in wave order;
-// splits meet through fp32 partial rows and a per-group counter exactly as in the
-// small-batch layer kernel: the workgroup that arrives last adds the partial rows
-// in split order, rounds to fp16 (ponyexl3/ref/forward.py:41), applies the output
+// matrix instructions; a wave stages exactly the activations it reads, so the
+// main loop has no workgroup barrier. The waves' sums are added through LDS as
+// (wave 0 + wave 1) + (wave 2 + wave 3); splits meet through fp32 partial rows
+// and a per-group counter exactly as in the small-batch layer kernel: the
+// workgroup that arrives last adds the partial rows in split order, rounds to fp16 (ponyexl3/ref/forward.py:41), applies the output
 // Hadamard, svh and bias. Counters must be zero on entry and are zero again on
 // exit.
 //
