@@ -81,13 +81,14 @@ class EXL3SwitchGLU(torch.nn.Module):
         )
 
     # The sorted, segmented prefill path replaces the per-slot kernels once the
-    # experts see a few rows each (the reference switches at 9 tokens,
+    # experts see about two rows each (the reference switches at 9 tokens,
     # ponyexl3/mlx/exl3_moe.py:770-787). Measured on 256 experts of 2048 x 512,
-    # top-8: the slot kernels cost ~4 us per token, the prefill path ~0.5 ms (every
-    # expert's weights are decoded once) plus ~0.15 us per token, so they cross near
-    # 128 tokens = 4 rows per expert.
+    # top-8: the slot kernels cost ~3.8 us per token (every slot reads its expert),
+    # the prefill path ~0.2 ms whatever the token count (every expert's weights are
+    # decoded once, eight launches); 48 tokens: 181 vs 197 us, 64 tokens: 253 vs
+    # 201 us, so they cross near 56 tokens = 1.75 rows per expert.
     prefill_min_tokens = 24
-    prefill_min_rows_per_expert = 4.0
+    prefill_min_rows_per_expert = 1.75
 
     def _use_prefill(self, tokens: int, top_k: int) -> bool:
         return (tokens >= self.prefill_min_tokens
