@@ -137,6 +137,31 @@ def test_config2_shapes_bs1(cuda, oracle, name, n_in, n_out):
     assert rel_l2(y[0], ref) <= TOL
 
 
+@pytest.mark.parametrize("name,n_in,n_out", [("k_proj", 5120, 1024), ("o_proj", 8192, 5120)])
+def test_config2_shapes_medium_batch(cuda, name, n_in, n_out):
+    """Config-2 shapes at 16 and 32 rows (batched decode): the medium-batch kernel
+    with its real split counts against the prefill GEMM on the same input (both
+    oracle-checked at small sizes; same fp32 products, other cut points) and, row by
+    row, against the one-row kernel (linearity of the layer in its batch rows)."""
+    from ponyexl3_amd import make_exl3_layer, ops
+
+    layer = make_exl3_layer(k=4, in_features=n_in, out_features=n_out, seed=20_016)
+    tr = ops.as_trellis_tensor(layer.trellis, cuda)
+    suh, svh = torch.from_numpy(layer.suh).to(cuda), torch.from_numpy(layer.svh).to(cuda)
+    rng = np.random.default_rng(16)
+    for rows in (16, 32):
+        _, xt = _x(rng, (rows, n_in), cuda)
+        print(f"config2 {name} rows={rows}", flush=True)
+        a = ops.linear_forward(xt, tr, 4, 0, suh, svh, fused=True)
+        b = ops.linear_forward(xt, tr, 4, 0, suh, svh, fused=False)
+        scale = float(b.float().abs().max())
+        assert float((a.float() - b.float()).abs().max()) <= 2e-3 * scale
+        for r in (0, rows - 1):
+            one = ops.linear_forward(xt[r : r + 1].contiguous(), tr, 4, 0, suh, svh, fused=True)
+            assert float((a[r : r + 1].float() - one.float()).abs().max()) <= 2e-3 * scale
+    assert int(ops.sync_counters(cuda, 1).abs().sum()) == 0
+
+
 @pytest.mark.parametrize("rows", [1, 8, 11, 16, 19])
 def test_fused_group_matches_members(cuda, oracle, rows):
     from ponyexl3_amd import EXL3Linear, FusedEXL3Group, make_exl3_layer
