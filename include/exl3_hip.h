@@ -96,20 +96,6 @@ int exl3_had128_pre(const uint16_t *x, int rows, int n, const uint16_t *suh, int
                     uint16_t *xh, void *stream);
 
 /*
- * Output-side Hadamard-128: optional split-K reduction, the fp16 cast of the
- * matmul result, the transform, svh and bias:
- *   t   = fp16( sum_{i < n_sum} y[i][r][:] )      (ponyexl3/ref/forward.py:41)
- *   out = fp16( had128(t) * svh ) (+ bias, fp16 add)  (ponyexl3/ref/forward.py:42-45)
- * Replaces EXL3LayerRuntime.finish_y (ponyexl3/mlx/layer_state.py:138-141),
- * _fused_finish (ponyexl3/mlx/exl3_fused.py:63-76) and the partial-sum
- * reduction of ponyexl3/mlx/gemv_metal.py:1454-1457. Slices are added in index
- * order, so the result is deterministic.
- *   y           fp32 [n_sum][rows][n] (y_is_fp32 = 1, slice stride sum_stride
- *               elements) or fp16 [rows][n] (y_is_fp32 = 0, n_sum must be 1)
- *   svh, bias   fp16 [n] or NULL
- *   out         fp16 [rows][n]; may alias y when y is fp16
- */
-/*
  * Hadamard-128 with one scale vector per row (rows routed to different experts),
  * with the row gathers and the final scatter of the sorted MoE prefill folded in:
  *   post == 0: out[o(r)] = fp16(had128(x[i(r)] * scale[s(r)]))  (_rows_prep,
@@ -124,6 +110,20 @@ int exl3_had128_rows(const uint16_t *x, int rows, int n, const int32_t *in_index
                      const uint16_t *scale, const int32_t *scale_index, size_t scale_ld, int post,
                      uint16_t *out, const int32_t *out_index, void *stream);
 
+/*
+ * Output-side Hadamard-128: optional split-K reduction, the fp16 cast of the
+ * matmul result, the transform, svh and bias:
+ *   t   = fp16( sum_{i < n_sum} y[i][r][:] )      (ponyexl3/ref/forward.py:41)
+ *   out = fp16( had128(t) * svh ) (+ bias, fp16 add)  (ponyexl3/ref/forward.py:42-45)
+ * Replaces EXL3LayerRuntime.finish_y (ponyexl3/mlx/layer_state.py:138-141),
+ * _fused_finish (ponyexl3/mlx/exl3_fused.py:63-76) and the partial-sum
+ * reduction of ponyexl3/mlx/gemv_metal.py:1454-1457. Slices are added in index
+ * order, so the result is deterministic.
+ *   y           fp32 [n_sum][rows][n] (y_is_fp32 = 1, slice stride sum_stride
+ *               elements) or fp16 [rows][n] (y_is_fp32 = 0, n_sum must be 1)
+ *   svh, bias   fp16 [n] or NULL
+ *   out         fp16 [rows][n]; may alias y when y is fp16
+ */
 int exl3_had128_post(const void *y, int y_is_fp32, int n_sum, size_t sum_stride, int rows, int n,
                      const uint16_t *svh, const uint16_t *bias, uint16_t *out, void *stream);
 
