@@ -39,6 +39,7 @@ extern "C" {
 #define EXL3_E_LAUNCH (-6)        /* hipGetLastError() was not hipSuccess after a launch */
 #define EXL3_E_BAD_INDEX (-7)     /* tile_sub / expert index table inconsistent */
 #define EXL3_E_UNSUPPORTED (-8)   /* valid request this build has no kernel for */
+#define EXL3_E_STATIC_LIMIT (-9)  /* exl3_linear_forward_static: beyond its built-in scratch */
 
 /* Library version (major*10000 + minor*100 + patch). */
 int exl3_version(void);
@@ -242,6 +243,29 @@ int exl3_linear_forward(const uint16_t *x, int rows, const uint16_t *trellis, in
                         size_t counters_len, void *stream);
 
 size_t exl3_linear_workspace_bytes(int rows, int in_features, int out_features, int n_sub);
+
+/*
+ * exl3_linear_forward for callers that cannot allocate device memory or carry a
+ * workspace: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc. It has no counterpart in the reference. Same arguments and
+ * results as exl3_linear_forward with counters (the one-launch kernel), minus
+ * workspace and counters: the split-K partial rows and the group counters live in
+ * a device array inside the library (exl3_linear_static_scratch_bytes() = 16 MiB of
+ * partial rows plus 4096 counters; every GPU the library runs on holds its copy
+ * until the process ends). No hipMalloc, hipFree or other allocating call is made.
+ *   rows <= exl3_gemv_max_rows(), otherwise EXL3_E_UNSUPPORTED;
+ *   exl3_linear_static_need_bytes(rows, in, out) must not exceed the scratch size
+ *   and out/128 must not exceed 4096, otherwise EXL3_E_STATIC_LIMIT (nothing is
+ *   launched).
+ * All calls on one GPU share that GPU's array: calls that overlap there (two
+ * streams, two threads) race. The counters are zero whenever no call is running.
+ */
+size_t exl3_linear_static_scratch_bytes(void);
+size_t exl3_linear_static_need_bytes(int rows, int in_features, int out_features);
+int exl3_linear_forward_static(const uint16_t *x, int rows, const uint16_t *trellis, int in_tiles,
+                               int out_tiles, int K, int cb, const uint16_t *suh, int n_sub,
+                               const int32_t *group_sub, const uint16_t *svh, const uint16_t *bias,
+                               uint16_t *y, void *stream);
 
 /*
  * Routed MoE expert chain for rows <= 8 tokens (EXL3SwitchGLU.__call__,

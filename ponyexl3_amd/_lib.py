@@ -22,6 +22,7 @@ EXL3_E_WORKSPACE = -5
 EXL3_E_LAUNCH = -6
 EXL3_E_BAD_INDEX = -7
 EXL3_E_UNSUPPORTED = -8
+EXL3_E_STATIC_LIMIT = -9
 
 _vp = ctypes.c_void_p
 _i = ctypes.c_int
@@ -60,6 +61,11 @@ PROTOTYPES = {
         [_vp, _i, _vp, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _sz, _vp],
     ),
     "exl3_linear_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "exl3_linear_static_scratch_bytes": (_sz, []),
+    "exl3_linear_static_need_bytes": (_sz, [_i, _i, _i]),
+    "exl3_linear_forward_static": (
+        _i, [_vp, _i, _vp, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp],
+    ),
     "exl3_moe_forward": (
         _i,
         [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _sz, _vp,

@@ -3,6 +3,8 @@
 #include "exl3_device.hpp"
 #include "exl3_host.hpp"
 
+#include <mutex>
+
 namespace exl3 {
 
 // Workspace layout of exl3_linear_forward:
@@ -54,6 +56,8 @@ EXL3_EXPORT const char* exl3_status_string(int status) {
         case EXL3_E_LAUNCH: return "HIP kernel launch failed";
         case EXL3_E_BAD_INDEX: return "inconsistent group/expert index table";
         case EXL3_E_UNSUPPORTED: return "no kernel for this request";
+        case EXL3_E_STATIC_LIMIT:
+            return "request needs more scratch than the built-in array of exl3_linear_forward_static holds";
         default: return "unknown status";
     }
 }
@@ -166,4 +170,89 @@ EXL3_EXPORT int exl3_linear_prefill(const uint16_t* xh, int rows, int n_sub, con
         return rc;
     if (post_done) return EXL3_OK;
     return launch_had_post(ytmp, 0, 1, 0, rows, out_features, svh, bias, y, s);
+}
+
+// ---------------------------------------------------------------------------
+// exl3_linear_forward_static: the one-launch small-batch layer for callers that
+// cannot allocate device memory (code under HIP graph capture, serving loops,
+// harnesses that forbid hipMalloc). The split-K partial rows and the group
+// counters, which exl3_linear_forward takes from the caller, live in a
+// file-scope device array instead. Each GPU holds its own copy of the array at
+// its own address for the life of the process; the address is looked up once
+// per device and only that pointer is ever handed to a kernel (the array's name
+// is a host-side stand-in, not a device address).
+namespace exl3 {
+
+constexpr size_t kStaticCounterInts = 4096;              // 128-column groups: out <= 524288
+constexpr size_t kStaticPartialBytes = (size_t)16 << 20;  // fp32 split-K partial rows
+constexpr size_t kStaticScratchBytes = kStaticPartialBytes + kStaticCounterInts * sizeof(int32_t);
+constexpr int kStaticMaxDevices = 64;
+
+__global__ void static_zero_kernel(int32_t* p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+}  // namespace exl3
+
+static __device__ __align__(256) unsigned char scratch[exl3::kStaticScratchBytes];
+
+namespace exl3 {
+
+// Device address of this GPU's copy of `scratch` (resolved on first use, with that
+// device current); the counters in it are cleared once by a fill kernel on `stream`.
+static int static_scratch(hipStream_t stream, unsigned char** out) {
+    static unsigned char* ptrs[kStaticMaxDevices];  // zero-initialised; one slot per device
+    static std::mutex lock;
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kStaticMaxDevices)
+        return EXL3_E_LAUNCH;
+    std::lock_guard<std::mutex> guard(lock);
+    if (!ptrs[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return EXL3_E_LAUNCH;
+        int32_t* counters = reinterpret_cast<int32_t*>(static_cast<unsigned char*>(p) + kStaticPartialBytes);
+        static_zero_kernel<<<dim3((unsigned)((kStaticCounterInts + 255) / 256)), dim3(256), 0, stream>>>(
+            counters, (int)kStaticCounterInts);
+        if (int rc = launch_status()) return rc;
+        ptrs[dev] = static_cast<unsigned char*>(p);
+    }
+    *out = ptrs[dev];
+    return EXL3_OK;
+}
+
+}  // namespace exl3
+
+EXL3_EXPORT size_t exl3_linear_static_scratch_bytes(void) { return exl3::kStaticPartialBytes; }
+
+EXL3_EXPORT size_t exl3_linear_static_need_bytes(int rows, int in_features, int out_features) {
+    using namespace exl3;
+    if (rows < 1 || rows > kLinearSmallMaxRows || in_features < 128 || out_features < 128) return 0;
+    const GemvPlan plan = plan_linear_small(rows, in_features / 16, out_features / 128);
+    return (size_t)plan.n_partials() * rows * out_features * sizeof(float);
+}
+
+EXL3_EXPORT int exl3_linear_forward_static(const uint16_t* x, int rows, const uint16_t* trellis,
+                                           int in_tiles, int out_tiles, int K, int cb,
+                                           const uint16_t* suh, int n_sub, const int32_t* group_sub,
+                                           const uint16_t* svh, const uint16_t* bias, uint16_t* y,
+                                           void* stream) {
+    using namespace exl3;
+    if (int rc = check_k_cb(K, cb)) return rc;
+    if (!x || !trellis || !y) return EXL3_E_NULL_POINTER;
+    if (rows < 1 || in_tiles < 8 || out_tiles < 8 || in_tiles % 8 || out_tiles % 8 || n_sub < 1)
+        return EXL3_E_BAD_SHAPE;
+    if (rows > kLinearSmallMaxRows) return EXL3_E_UNSUPPORTED;  // only the one-launch kernel
+    if (n_sub > 1 && (!group_sub || !suh)) return EXL3_E_BAD_INDEX;
+    const int n_groups = out_tiles / 8;
+    if ((size_t)n_groups > kStaticCounterInts) return EXL3_E_STATIC_LIMIT;
+    const GemvPlan plan = plan_linear_small(rows, in_tiles, n_groups);
+    const size_t need = (size_t)plan.n_partials() * rows * out_tiles * 16 * sizeof(float);
+    if (need > kStaticPartialBytes) return EXL3_E_STATIC_LIMIT;
+    hipStream_t s = as_stream(stream);
+    unsigned char* base = nullptr;
+    if (int rc = static_scratch(s, &base)) return rc;
+    return launch_linear_small(x, rows, trellis, in_tiles, out_tiles, K, cb, suh, n_sub, group_sub,
+                               svh, bias, y, reinterpret_cast<float*>(base),
+                               reinterpret_cast<int*>(base + kStaticPartialBytes), plan, s);
 }

@@ -1,0 +1,99 @@
+"""exl3_linear_forward_static (the entry point that allocates nothing) against
+exl3_linear_forward with caller-owned workspace and counters: same kernel, so the
+outputs must be bit-identical; two calls in a row, the second on a smaller input,
+because every call on a GPU shares one built-in scratch array."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _layer_tensors(cuda, k, n_in, n_out, seed, mcg=False, bias=False):
+    from ponyexl3_amd import make_exl3_layer
+    from ponyexl3_amd.ops import as_trellis_tensor
+
+    layer = make_exl3_layer(k=k, in_features=n_in, out_features=n_out, seed=seed, mcg=mcg, bias=bias)
+    t = as_trellis_tensor(layer.trellis, cuda)
+    suh = torch.from_numpy(layer.suh).to(cuda)
+    svh = torch.from_numpy(layer.svh).to(cuda)
+    b = torch.from_numpy(layer.bias).to(cuda) if bias else None
+    return layer, t, suh, svh, b
+
+
+def _forward_pair(lib, cuda, x, t, k, cb, suh, svh, bias):
+    """(reference entry point, static entry point) outputs for one layer."""
+    from ponyexl3_amd import _lib as L
+
+    rows, n_in = x.shape
+    in_tiles, out_tiles = t.shape[0], t.shape[1]
+    n_out = out_tiles * 16
+    ws_bytes = int(lib.exl3_linear_workspace_bytes(rows, n_in, n_out, 1))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
+    cnt = torch.zeros(n_out // 128, dtype=torch.int32, device=cuda)
+    y_ref = torch.empty((rows, n_out), dtype=torch.float16, device=cuda)
+    rc = lib.exl3_linear_forward(_ptr(x), rows, _ptr(t), in_tiles, out_tiles, k, cb, _ptr(suh), 1, None,
+                                 _ptr(svh), _ptr(bias), _ptr(y_ref), _ptr(ws), ws.numel(), _ptr(cnt),
+                                 cnt.numel(), _stream())
+    L.check(rc, "exl3_linear_forward")
+    y = torch.full((rows, n_out), float("nan"), dtype=torch.float16, device=cuda)
+    rc = lib.exl3_linear_forward_static(_ptr(x), rows, _ptr(t), in_tiles, out_tiles, k, cb, _ptr(suh), 1,
+                                        None, _ptr(svh), _ptr(bias), _ptr(y), _stream())
+    L.check(rc, "exl3_linear_forward_static")
+    torch.cuda.synchronize()
+    assert int(cnt.abs().sum()) == 0
+    return y_ref.cpu().numpy(), y.cpu().numpy()
+
+
+def test_static_entry_matches_workspace_entry_twice(cuda, oracle):
+    from ponyexl3_amd import _lib as L
+    from conftest import rel_l2
+
+    lib = L.load()
+    assert int(lib.exl3_linear_static_scratch_bytes()) == 16 << 20
+    rng = np.random.default_rng(5)
+    # first call: many split partial rows (2176 x 640, 4 rows); second: a smaller layer, 1 row
+    for (k, mcg, n_in, n_out, rows, seed) in [(4, False, 2176, 640, 4, 3), (3, True, 256, 384, 1, 4)]:
+        print(f"static entry k={k} mcg={mcg} {n_in}x{n_out} rows={rows}", flush=True)
+        layer, t, suh, svh, b = _layer_tensors(cuda, k, n_in, n_out, seed, mcg=mcg, bias=True)
+        xn = rng.standard_normal((rows, n_in)).astype(np.float16)
+        x = torch.from_numpy(xn).to(cuda)
+        need = int(lib.exl3_linear_static_need_bytes(rows, n_in, n_out))
+        assert 0 < need <= 16 << 20
+        y_ref, y = _forward_pair(lib, cuda, x, t, k, 1 if mcg else 0, suh, svh, b)
+        assert np.array_equal(y.view(np.uint16), y_ref.view(np.uint16))
+        want = oracle.linear_forward(layer.trellis, layer.k, layer.codebook_mode, layer.suh, layer.svh, xn,
+                                     bias=layer.bias)
+        assert rel_l2(y, want) <= 1e-3
+
+
+def test_static_entry_rejects_what_does_not_fit(cuda):
+    from ponyexl3_amd import _lib as L
+
+    lib = L.load()
+    x = torch.zeros((9, 256), dtype=torch.float16, device=cuda)
+    t = torch.zeros((16, 16, 64), dtype=torch.int16, device=cuda)
+    y = torch.zeros((9, 256), dtype=torch.float16, device=cuda)
+    # more rows than the one-launch kernel takes
+    rc = lib.exl3_linear_forward_static(_ptr(x), 9, _ptr(t), 16, 16, 4, 0, None, 1, None, None, None,
+                                        _ptr(y), _stream())
+    assert rc == L.EXL3_E_UNSUPPORTED
+    # a shape whose partial rows exceed the built-in scratch: only sizes are looked at,
+    # so the (too small) buffers are never touched
+    in_tiles, out_tiles = 4096, 65536
+    assert int(lib.exl3_linear_static_need_bytes(8, in_tiles * 16, out_tiles * 16)) > 16 << 20
+    rc = lib.exl3_linear_forward_static(_ptr(x), 8, _ptr(t), in_tiles, out_tiles, 4, 0, None, 1, None,
+                                        None, None, _ptr(y), _stream())
+    assert rc == L.EXL3_E_STATIC_LIMIT
+    assert "built-in" in L.status_string(rc)
+    torch.cuda.synchronize()
