@@ -15,9 +15,12 @@ whole step (Hadamard kernels and launch gaps included).
 Prints ONE JSON line: metric, value, unit, n_gpus, steps, warmup, ms_per_step,
 higher_is_better, scaling, vs_baseline, dtype, data, config, plus the objects
 roofline (dominant kernel = the one-launch layer kernel, launch durations from
-HIP events around batched graph replays on cold weights), cpu_baseline (the C
+HIP events around batched graph replays on cold weights; next to the published
+8 TB/s it carries the streaming-read rate and the decode-loop rate measured in
+the same run), ceilings (those two measurements in full), cpu_baseline (the C
 oracle on the host cores), batch_rows (2..128 rows), config1, prefill_gemm
-(M=2048, config 3), moe (config 4) and, with --sweep, config5.
+(M=2048, config 3), moe (config 4), encoder and config5 (K in {2,6,8}, 3INST and
+MCG, 1 and 8 rows; --sweep: K in {2,3,5,6,8} at 1/4/8 rows).
 """
 
 from __future__ import annotations
@@ -161,6 +164,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--repeats", type=int, default=7,
+                    help="the timed region of --steps steps is run this many times; the median is reported")
     ap.add_argument("--layers", type=int, default=4, help="distinct weight copies rotated over")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
     ap.add_argument("--skip-cpu", action="store_true")
@@ -257,11 +262,17 @@ def main():
 
     run_steps(args.warmup)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    run_steps(args.steps)
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    # exactly --steps steps between two synchronisations, --repeats times; the
+    # reported figure is the median of the repeats (a 20-step region is under 2 ms)
+    samples = []
+    for _ in range(max(1, args.repeats)):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run_steps(args.steps)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        samples.append((t1 - t0) * 1e3 / args.steps)
+    ms_per_step = float(np.median(samples))
     value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
 
     # ---- roofline of the dominant kernel: the one-launch layer kernel (input
@@ -290,18 +301,28 @@ def main():
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
         "traffic": TRAFFIC_BYTES_PER_STEP,
+        "traffic_source": "profiles/linear_small_k4_config2_pmc.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this "
+                          "script, scaled by a 64 MiB copy); a constant, not measured in this run",
         "bytes_per_launch": "in*out*K/8 of the launch's linear(s); achieved = sum over the launches of a step / "
                             "sum of their mean durations; traffic = HBM bytes of the same launches (FETCH_SIZE + WRITE_SIZE)",
         "per_linear": per_linear,
     }
 
-    extras = {}
+    ceilings = bench_ceilings(dev)
+    roofline["measured_peak"] = ceilings["stream_read_GBps"]
+    roofline["frac_of_measured_peak"] = round(achieved / ceilings["stream_read_GBps"], 4)
+    roofline["decode_loop_ceiling_GBps"] = ceilings["decode_loop"]["k4_3inst_cold"]["GBps"]
+    roofline["frac_of_decode_loop_ceiling"] = round(
+        achieved / ceilings["decode_loop"]["k4_3inst_cold"]["GBps"], 4)
+    extras = {"ceilings": ceilings}
     if not args.skip_extras:
         extras.update(bench_batch_rows(dev, layers[0]))
         extras.update(bench_config1(dev))
         extras.update(bench_prefill(dev, layers[0], xs))
         extras.update(bench_moe(dev))
         extras.update(bench_encoder(dev))
+        if not args.sweep:
+            extras.update(bench_sweep(dev, layers[0], ks=(2, 6, 8), row_counts=(1, 8)))
     if args.sweep:
         extras.update(bench_sweep(dev, layers[0]))
 
@@ -314,6 +335,7 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5),
+        "ms_per_step_samples": [round(v, 5) for v in samples],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -402,6 +424,72 @@ def _rows_x(n, rows, dev):
     return torch.randn((rows, n), generator=g).to(torch.float16).to(dev)
 
 
+def bench_ceilings(dev):
+    """What this GPU delivers, measured in the same run: a streaming read of cold
+    memory (the denominator next to the published 8 TB/s), and the small-batch
+    kernels' inner loop on its own (wave-wide load, per-lane decode of 32 codewords,
+    8 matrix-pipe dot products; one workgroup of 16 waves per CU, 128 tile rows per
+    wave, no Hadamard, no reduction): the rate the VALU instruction sequence of the
+    bit-exact decode allows before any layer structure is added. 'cold' walks over a
+    2 GiB buffer so that every launch reads memory no earlier launch of the
+    measurement touched; 'cache' re-reads one 32 MiB slice."""
+    import ctypes
+
+    import torch
+
+    from ponyexl3_amd import _lib
+
+    lib = _lib.load()
+    total = 2 << 30
+    buf = torch.randint(-2**31, 2**31 - 1, (total // 4,), dtype=torch.int32, device=dev)
+    out = torch.zeros(4096 * 1024, dtype=torch.float32, device=dev)
+    stream = lambda: ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ptr = lambda off: ctypes.c_void_p(buf.data_ptr() + off)
+    n_cu = torch.cuda.get_device_properties(dev).multi_processor_count
+
+    def timed(launches):
+        """mean ms per launch of a list of launch thunks, run back to back twice
+        (first pass warms code and TLBs) between two events"""
+        for fn in launches:
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for fn in launches:
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / len(launches)
+
+    chunk = 512 << 20
+    read = [(lambda o=o: _lib.check(lib.exl3_diag_stream_read(ptr(o), chunk, ctypes.c_void_p(out.data_ptr()), stream()),
+                                    "exl3_diag_stream_read")) for o in range(0, total, chunk)]
+    ms = timed(read)
+    res = {"stream_read_GBps": round(chunk / ms / 1e6, 1), "stream_read_chunk_MB": chunk >> 20,
+           "published_peak_GBps": HBM_PEAK_GBS}
+    steps = 128
+    loops = {}
+    for tag, k, cb, cold in (("k4_3inst_cold", 4, 0, True), ("k4_3inst_cache", 4, 0, False),
+                             ("k4_mcg_cold", 4, 1, True), ("k2_3inst_cold", 2, 0, True),
+                             ("k8_3inst_cold", 8, 0, True)):
+        per_launch = n_cu * 16 * steps * 256 * k  # bytes one launch walks over
+        offs = list(range(0, total - per_launch + 1, per_launch)) if cold else [0] * 8
+        size = per_launch if cold else 32 << 20
+        calls = [(lambda o=o: _lib.check(lib.exl3_diag_decode_loop(ptr(o), size, k, cb, n_cu, steps,
+                                                                     ctypes.c_void_p(out.data_ptr()), stream()),
+                                         "exl3_diag_decode_loop")) for o in offs]
+        ms = timed(calls)
+        weights = n_cu * 16 * steps * 2048
+        loops[tag] = {"us_per_launch": round(ms * 1e3, 1), "Tweights_per_s": round(weights / ms / 1e9, 2),
+                      "GBps": round(weights * k / 8 / ms / 1e6, 1),
+                      "frac_hbm_peak": round(weights * k / 8 / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    res["decode_loop"] = loops
+    res["decode_loop_note"] = ("n_cu workgroups x 16 waves x 128 tile rows per launch, launch overhead included "
+                               "(about 10 % of a launch)")
+    del buf, out
+    return res
+
+
 def bench_batch_rows(dev, layer):
     """The same layer step at 2 .. 128 rows (batched decode, speculative verify):
     sum of the launch durations on cold weights (9..32 rows: each linear is the
@@ -423,13 +511,14 @@ def bench_config1(dev):
                         "GBps": round(lin.bytes / ms / 1e6, 1)}}
 
 
-def bench_sweep(dev, layer):
-    """config 5: the config-2 layer at other bit widths and codebooks, 1/4/8 rows."""
+def bench_sweep(dev, layer, ks=(2, 3, 5, 6, 8), row_counts=(1, 4, 8)):
+    """config 5: the config-2 layer at other bit widths and codebooks (the default run
+    takes K in {2, 6, 8} at 1 and 8 rows, --sweep all of K in {2,3,5,6,8} at 1/4/8)."""
     res = {}
-    for k in (2, 3, 5, 6, 8):
+    for k in ks:
         total = sum(l.n_in * l.n_out * k // 8 for l in layer)
         for cb, cbn in ((0, "3inst"), (1, "mcg")):
-            for rows in (1, 4, 8):
+            for rows in row_counts:
                 ms = sum(_launch_ms(lin, _rows_x(lin.n_in, rows, dev), k, dev, cb=cb) for lin in layer)
                 res[f"k{k}_{cbn}_rows{rows}"] = {"us_per_step": round(ms * 1e3, 2),
                                                  "GBps": round(total / ms / 1e6, 1)}

@@ -47,6 +47,22 @@ int exl3_version(void);
 /* Human-readable text for a status code; never NULL. */
 const char *exl3_status_string(int status);
 
+/*
+ * Diagnostics for measured ceilings (no counterpart in the reference; its kernel
+ * benches quote Gw/s only, tools/bench/gemv_split_bench.py:51,84).
+ * exl3_diag_stream_read: reads `bytes` (16-byte aligned buffer) once with streaming
+ *   loads; out: 4 bytes of device memory, practically never written.
+ * exl3_diag_decode_loop: n_wg workgroups of 16 waves run `steps` (a multiple of 4)
+ *   iterations of the small-batch kernels' inner loop (one wave-wide load of 256*K
+ *   bytes, per-lane decode of 32 codewords, 8 matrix-pipe dot products) over
+ *   consecutive 256*K-byte rows of buf, wrapping at the largest power-of-two row
+ *   count that fits in `bytes`; weights per launch = n_wg*16*steps*2048. cb 0 or 1.
+ *   out: float [n_wg*1024].
+ */
+int exl3_diag_stream_read(const void *buf, size_t bytes, void *out, void *stream);
+int exl3_diag_decode_loop(const void *buf, size_t bytes, int K, int cb, int n_wg, int steps,
+                          float *out, void *stream);
+
 /* Largest row count the small-batch kernel (exl3_gemv) accepts per call. */
 int exl3_gemv_max_rows(void);
 

@@ -19,7 +19,7 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(PKG_DIR, "libexl3_hip.so")
 
-SOURCES = ["decode.hip", "hadamard.hip", "gemv.hip", "linear_mid.hip", "gemm.hip", "moe.hip", "search.hip", "capi.hip"]
+SOURCES = ["decode.hip", "hadamard.hip", "gemv.hip", "linear_mid.hip", "gemm.hip", "moe.hip", "search.hip", "diag.hip", "capi.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
