@@ -1,10 +1,13 @@
 """Converted-checkpoint reader: ``quantization_config.json`` + safetensors ->
 ``EXL3Layer`` objects, expert stacking and the sibling-fusion policy.
 
-Host-side only (numpy + safetensors; torch is touched where modules are built).
-Mirrors ``ponyexl3/ref/loader.py:41-173`` (same function names, same errors) and
-the module-building helpers of ``ponyexl3/mlx/model.py``: the multiplier check
-(:261-283), expert stacking (:77-127) and the fusion policy (:325-432).
+Host-side only (numpy; torch is touched where modules are built). A model
+directory is scanned once into a ``Checkpoint``: the EXL3 records of the config and
+a tensor-name -> shard table from the index file or the shard headers; tensors are
+views into memory-mapped shards. The module-level functions keep the names of
+``ponyexl3/ref/loader.py:41-173``; the module-building helpers follow
+``ponyexl3/mlx/model.py``: multiplier check (:261-283), expert stacking (:77-127),
+fusion policy (:325-432).
 
 On-disk schema per module key (``ponyexl3/convert/discovery.py:191-212``):
 ``{key}.trellis`` int16 ``(in/16, out/16, 16K)`` (reinterpreted as uint16),
@@ -18,9 +21,11 @@ holding the codebook multiplier, and in ``quantization_config.json`` the
 from __future__ import annotations
 
 import json
+import mmap
 import os
-from glob import glob
-from typing import Any
+import struct
+from dataclasses import asdict, dataclass
+from typing import Any, Iterator
 
 import numpy as np
 
@@ -29,162 +34,228 @@ from .layer import EXL3Layer
 MCG_MULT = 0xCBAC1FED  # ponyexl3/ref/codebook.py:19-20
 MUL1_MULT = 0x83DCD12D
 
-_WEIGHT_INDEX_CACHE: dict[str, dict[str, str] | None] = {}
+# safetensors dtype tag -> numpy dtype, for the tensors an EXL3 module stores
+_ST_DTYPES = {"I16": np.int16, "U16": np.uint16, "F16": np.float16, "F32": np.float32,
+              "I32": np.int32, "U32": np.uint32, "I64": np.int64, "U8": np.uint8, "I8": np.int8}
+
+
+class _Shard:
+    """One .safetensors file: 8-byte little-endian header length, a JSON header
+    {name: {dtype, shape, data_offsets}}, then the raw tensor bytes. The header is
+    parsed once; tensors are read-only views into one memory map of the file."""
+
+    def __init__(self, path: str):
+        self.path = path
+        with open(path, "rb") as f:
+            (hlen,) = struct.unpack("<Q", f.read(8))
+            header = json.loads(f.read(hlen))
+        header.pop("__metadata__", None)
+        self.entries: dict[str, dict] = header
+        self._base = 8 + hlen
+        self._map: mmap.mmap | None = None
+
+    def names(self) -> Iterator[str]:
+        return iter(self.entries)
+
+    def tensor(self, name: str) -> np.ndarray:
+        e = self.entries[name]
+        dt = _ST_DTYPES.get(e["dtype"])
+        if dt is None:
+            raise ValueError(f"{self.path}: tensor {name!r} has unsupported dtype {e['dtype']}")
+        if self._map is None:
+            with open(self.path, "rb") as f:
+                self._map = mmap.mmap(f.fileno(), 0, access=mmap.ACCESS_READ)
+        lo, hi = e["data_offsets"]
+        n = int(np.prod(e["shape"], dtype=np.int64)) if e["shape"] else 1
+        if hi - lo != n * np.dtype(dt).itemsize:
+            raise ValueError(f"{self.path}: tensor {name!r} has {hi - lo} bytes for shape {e['shape']}")
+        return np.frombuffer(self._map, dtype=dt, count=n, offset=self._base + lo).reshape(e["shape"])
+
+
+@dataclass(frozen=True)
+class LayerMeta:
+    """Dimensions of one EXL3 module as recorded in quantization_config.json."""
+
+    key: str
+    k: int
+    bits_per_weight: Any
+    in_features: int
+    out_features: int
+    in_tiles: int
+    out_tiles: int
+    n_tiles: int
+    trellis_shape: tuple
+    trellis_bytes: int
+    weight_fp16_bytes: int
+    mcg: bool
+    mul1: bool
+
+    def __getitem__(self, name: str):  # meta["k"], as callers of the reference's dict expect
+        return getattr(self, name)
+
+    def as_dict(self) -> dict[str, Any]:
+        return asdict(self)
+
+
+class Checkpoint:
+    """A converted model directory, scanned once: the EXL3 records of
+    quantization_config.json and a tensor-name -> shard table built from
+    model.safetensors.index.json or, without one, from the headers of every
+    *.safetensors file below the directory. Shards stay mapped while the object lives."""
+
+    def __init__(self, model_dir: str):
+        self.model_dir = model_dir
+        qpath = os.path.join(model_dir, "quantization_config.json")
+        if not os.path.isfile(qpath):
+            raise FileNotFoundError(f"no quantization_config.json in {model_dir}")
+        with open(qpath, encoding="utf-8") as f:
+            storage = json.load(f).get("tensor_storage", {})
+        self.records: dict[str, dict] = {key: rec for key, rec in storage.items()
+                                         if rec.get("quant_format") == "exl3"}
+        self._shards: dict[str, _Shard] = {}
+        self._where: dict[str, str] = {}
+        index = os.path.join(model_dir, "model.safetensors.index.json")
+        listed: dict[str, str] = {}
+        if os.path.isfile(index):
+            with open(index, encoding="utf-8") as f:
+                listed = json.load(f).get("weight_map", {})
+        for name, rel in listed.items():
+            path = os.path.join(model_dir, rel)
+            if os.path.isfile(path):
+                self._where[name] = path
+        if len(self._where) < len(listed) or not listed:
+            # no index, or one that names files that are not there: read the headers
+            for root, _dirs, files in sorted(os.walk(model_dir)):
+                for fn in sorted(files):
+                    if fn.endswith(".safetensors"):
+                        shard = self._shard(os.path.join(root, fn))
+                        for name in shard.names():
+                            self._where.setdefault(name, shard.path)
+
+    def _shard(self, path: str) -> _Shard:
+        if path not in self._shards:
+            self._shards[path] = _Shard(path)
+        return self._shards[path]
+
+    def has(self, tensor_name: str) -> bool:
+        path = self._where.get(tensor_name)
+        return path is not None and tensor_name in self._shard(path).entries
+
+    def tensor(self, tensor_name: str) -> np.ndarray | None:
+        """A copy of the stored tensor, or None when no shard holds it."""
+        if not self.has(tensor_name):
+            return None
+        return np.array(self._shard(self._where[tensor_name]).tensor(tensor_name))
+
+    def keys(self) -> list[str]:
+        return sorted(self.records)
+
+    def meta(self, key: str) -> LayerMeta:
+        rec = self.records.get(key)
+        if rec is None:
+            raise KeyError(f"quantization_config.json has no EXL3 record for {key!r}")
+        stored = rec.get("stored_tensors", {})
+        entry = stored.get(f"{key}.trellis")
+        if entry is None:
+            raise KeyError(f"record of {key!r} lists no trellis tensor")
+        in_tiles, out_tiles, packed = (int(v) for v in entry["shape"])
+        return LayerMeta(
+            key=key, k=packed // 16, bits_per_weight=rec.get("bits_per_weight"),
+            in_features=16 * in_tiles, out_features=16 * out_tiles, in_tiles=in_tiles,
+            out_tiles=out_tiles, n_tiles=in_tiles * out_tiles,
+            trellis_shape=(in_tiles, out_tiles, packed), trellis_bytes=int(entry.get("n_bytes", 0)),
+            weight_fp16_bytes=in_tiles * out_tiles * 256 * 2, mcg=bool(rec.get("mcg_multiplier")),
+            mul1=bool(rec.get("mul1_multiplier")))
+
+    def check_multiplier(self, key: str, name: str, expected: int) -> None:
+        stored = self.tensor(f"{key}.{name}")
+        if stored is None:
+            return  # older checkpoints carry only the flag
+        got = int(stored.astype(np.int64).ravel()[0]) & 0xFFFFFFFF
+        if got != int(expected):
+            raise ValueError(f"{key}: the checkpoint was quantized with {name} multiplier {got:#010x}; "
+                             f"the kernels implement {int(expected):#010x} only")
+
+    def layer(self, key: str) -> EXL3Layer:
+        meta = self.meta(key)
+        trellis = self.tensor(f"{key}.trellis")
+        if trellis is None:
+            raise FileNotFoundError(f"{key}.trellis is listed in quantization_config.json but in no shard")
+        if trellis.dtype.itemsize != 2 or trellis.dtype.kind not in "iu":
+            raise ValueError(f"{key}.trellis must be a 16-bit integer tensor, found {trellis.dtype}")
+        if meta.mcg:
+            self.check_multiplier(key, "mcg", MCG_MULT)
+        if meta.mul1:
+            self.check_multiplier(key, "mul1", MUL1_MULT)
+
+        def first(*names):
+            for n in names:
+                t = self.tensor(f"{key}.{n}")
+                if t is not None:
+                    return t
+            return None
+
+        layer = EXL3Layer(key=key, in_features=meta.in_features, out_features=meta.out_features,
+                          k=meta.k, trellis=trellis.view(np.uint16), suh=first("suh", "su"),
+                          svh=first("svh", "sv"), bias=first("bias"), mcg=meta.mcg, mul1=meta.mul1)
+        layer.validate()
+        return layer
+
+
+_CHECKPOINTS: dict[str, Checkpoint] = {}
+
+
+def open_checkpoint(model_dir: str) -> Checkpoint:
+    """The (cached) scan of a model directory."""
+    ck = _CHECKPOINTS.get(model_dir)
+    if ck is None:
+        ck = _CHECKPOINTS[model_dir] = Checkpoint(model_dir)
+    return ck
 
 
 def clear_weight_index_cache(model_dir: str) -> None:
-    """Drop the cached safetensors index for a model directory."""
-    _WEIGHT_INDEX_CACHE.pop(model_dir, None)
-
-
-def _weight_index(model_dir: str) -> dict[str, str] | None:
-    if model_dir not in _WEIGHT_INDEX_CACHE:
-        path = os.path.join(model_dir, "model.safetensors.index.json")
-        if os.path.isfile(path):
-            with open(path, encoding="utf-8") as f:
-                _WEIGHT_INDEX_CACHE[model_dir] = json.load(f).get("weight_map", {})
-        else:
-            _WEIGHT_INDEX_CACHE[model_dir] = None
-    return _WEIGHT_INDEX_CACHE[model_dir]
+    """Forget the scan of a model directory (its files changed)."""
+    _CHECKPOINTS.pop(model_dir, None)
 
 
 def list_exl3_layers(model_dir: str) -> list[dict[str, Any]]:
-    """EXL3 linear modules named by quantization_config.json, sorted by key."""
-    qpath = os.path.join(model_dir, "quantization_config.json")
-    if not os.path.isfile(qpath):
-        raise FileNotFoundError(f"missing {qpath}")
-    with open(qpath, encoding="utf-8") as f:
-        qcfg = json.load(f)
-    layers = []
-    for key, info in qcfg.get("tensor_storage", {}).items():
-        if info.get("quant_format") != "exl3":
-            continue
-        layers.append({
-            "key": key,
-            "bits_per_weight": info.get("bits_per_weight"),
-            "stored_tensors": info.get("stored_tensors", {}),
-            "mcg": bool(info.get("mcg_multiplier")),
-            "mul1": bool(info.get("mul1_multiplier")),
-        })
-    return sorted(layers, key=lambda x: x["key"])
+    """One entry per EXL3 module of quantization_config.json, sorted by key
+    (the listing of ponyexl3/ref/loader.py:41-67)."""
+    ck = open_checkpoint(model_dir)
+    return [{"key": key, "bits_per_weight": ck.records[key].get("bits_per_weight"),
+             "stored_tensors": ck.records[key].get("stored_tensors", {}),
+             "mcg": bool(ck.records[key].get("mcg_multiplier")),
+             "mul1": bool(ck.records[key].get("mul1_multiplier"))} for key in ck.keys()]
 
 
-def layer_meta_from_config(model_dir: str, module_key: str) -> dict[str, Any]:
-    """Layer dimensions and on-disk sizes without loading weight tensors."""
-    meta = {x["key"]: x for x in list_exl3_layers(model_dir)}
-    if module_key not in meta:
-        raise KeyError(f"{module_key!r} not in quantization_config tensor_storage")
-    info = meta[module_key]
-    stored = info["stored_tensors"]
-    trellis_key = f"{module_key}.trellis"
-    if trellis_key not in stored:
-        raise KeyError(f"missing {trellis_key}")
-    shape = stored[trellis_key]["shape"]
-    in_tiles, out_tiles, packed_size = int(shape[0]), int(shape[1]), int(shape[2])
-    return {
-        "key": module_key,
-        "k": packed_size * 16 // 256,
-        "bits_per_weight": info.get("bits_per_weight"),
-        "in_features": in_tiles * 16,
-        "out_features": out_tiles * 16,
-        "in_tiles": in_tiles,
-        "out_tiles": out_tiles,
-        "n_tiles": in_tiles * out_tiles,
-        "trellis_shape": (in_tiles, out_tiles, packed_size),
-        "trellis_bytes": int(stored[trellis_key].get("n_bytes", 0)),
-        "weight_fp16_bytes": in_tiles * out_tiles * 512,
-        "mcg": info["mcg"],
-        "mul1": info["mul1"],
-    }
-
-
-def _find_shard(model_dir: str, tensor_key: str) -> str:
-    from safetensors import safe_open
-
-    index = _weight_index(model_dir)
-    if index is not None:
-        shard = index.get(tensor_key)
-        if shard is not None:
-            path = os.path.join(model_dir, shard)
-            if os.path.isfile(path):
-                return path
-    for pattern in (os.path.join(model_dir, "*.safetensors"),
-                    os.path.join(model_dir, "**", "*.safetensors")):
-        for path in sorted(glob(pattern, recursive=True)):
-            with safe_open(path, framework="np") as st:
-                if tensor_key in st.keys():
-                    return path
-    raise FileNotFoundError(f"tensor {tensor_key!r} not found under {model_dir}")
-
-
-def _load_tensor(model_dir: str, tensor_key: str) -> np.ndarray | None:
-    from safetensors import safe_open
-
-    try:
-        path = _find_shard(model_dir, tensor_key)
-    except FileNotFoundError:
-        return None
-    with safe_open(path, framework="np") as st:
-        return np.array(st.get_tensor(tensor_key))
+def layer_meta_from_config(model_dir: str, module_key: str) -> LayerMeta:
+    """Shapes and sizes of a module from the config alone; no tensor is read
+    (ponyexl3/ref/loader.py:70-103)."""
+    return open_checkpoint(model_dir).meta(module_key)
 
 
 def has_exl3_layer_weights(model_dir: str, module_key: str) -> bool:
-    """True when trellis weights exist on disk (vs a plan-only quantization_config)."""
-    try:
-        _find_shard(model_dir, f"{module_key}.trellis")
-    except FileNotFoundError:
-        return False
-    return True
+    """Whether a shard holds the module's trellis (a plan-only config lists modules
+    that were never written)."""
+    return open_checkpoint(model_dir).has(f"{module_key}.trellis")
 
 
 def check_multiplier(model_dir: str, module_key: str, name: str, expected: int) -> None:
-    """The codebooks hard-code the default multipliers; a checkpoint quantized with
-    another one must be refused rather than decoded to garbage
-    (``_check_multiplier``, ponyexl3/mlx/model.py:261-270). A missing scalar passes."""
-    t = _load_tensor(model_dir, f"{module_key}.{name}")
-    if t is None:
-        return
-    got = int(np.asarray(t).astype(np.int64).reshape(-1)[0]) & 0xFFFFFFFF
-    if got != int(expected):
-        raise ValueError(
-            f"{module_key}: stored {name} multiplier {got:#x} != supported {int(expected):#x}")
+    """The codebooks hard-code their multipliers; a checkpoint quantized with another
+    one is refused rather than decoded to garbage (ponyexl3/mlx/model.py:261-270)."""
+    open_checkpoint(model_dir).check_multiplier(module_key, name, expected)
 
 
 def load_exl3_layer(model_dir: str, module_key: str) -> EXL3Layer:
-    """Load one EXL3 linear layer by module key (e.g. model.layers.0.mlp.gate_proj)."""
-    if not has_exl3_layer_weights(model_dir, module_key):
-        raise FileNotFoundError(f"{module_key}.trellis")
-    cfg = layer_meta_from_config(model_dir, module_key)
-    trellis = _load_tensor(model_dir, f"{module_key}.trellis")
-    if trellis is None:
-        raise FileNotFoundError(f"{module_key}.trellis")
-    if trellis.dtype not in (np.uint16, np.int16):
-        raise ValueError(f"{module_key}.trellis has dtype {trellis.dtype}, expected int16/uint16")
-    if cfg["mcg"]:
-        check_multiplier(model_dir, module_key, "mcg", MCG_MULT)
-    if cfg["mul1"]:
-        check_multiplier(model_dir, module_key, "mul1", MUL1_MULT)
-    suh = _load_tensor(model_dir, f"{module_key}.suh")
-    if suh is None:
-        suh = _load_tensor(model_dir, f"{module_key}.su")
-    svh = _load_tensor(model_dir, f"{module_key}.svh")
-    if svh is None:
-        svh = _load_tensor(model_dir, f"{module_key}.sv")
-    bias = _load_tensor(model_dir, f"{module_key}.bias")
-    layer = EXL3Layer(
-        key=module_key, in_features=cfg["in_features"], out_features=cfg["out_features"],
-        k=cfg["k"], trellis=trellis.view(np.uint16), suh=suh, svh=svh, bias=bias,
-        mcg=cfg["mcg"], mul1=cfg["mul1"],
-    )
-    layer.validate()
-    return layer
+    """One EXL3 module by key, e.g. model.layers.0.mlp.gate_proj
+    (ponyexl3/ref/loader.py:138-173)."""
+    return open_checkpoint(model_dir).layer(module_key)
 
 
 def load_all_exl3_layers(model_dir: str) -> dict[str, EXL3Layer]:
-    """Every EXL3 module of the checkpoint whose weights are on disk, by key."""
-    return {info["key"]: load_exl3_layer(model_dir, info["key"])
-            for info in list_exl3_layers(model_dir)
-            if has_exl3_layer_weights(model_dir, info["key"])}
+    """Every EXL3 module whose trellis is on disk, by key."""
+    ck = open_checkpoint(model_dir)
+    return {key: ck.layer(key) for key in ck.keys() if ck.has(f"{key}.trellis")}
 
 
 # ---------------------------------------------------------------------------

@@ -8,20 +8,19 @@ identity through the same prefill forward the exact engine uses (input Hadamard
 kernel, MFMA trellis GEMM, output Hadamard kernel), one stripe of output columns
 at a time, so the folded weight carries exactly the runtime's cast points.
 
-The reference's w8a16 / w4a16 targets re-quantize W_pub with MLX's affine group
-quantizer (``native.py:88-124,216-264``); that is an MLX storage format with no
-counterpart here and is not provided.
+Only the fold itself is provided: it is the fp16 materialisation of the decode path.
+The reference's lossy engines around it (w8a16 / w4a16 re-quantization with MLX's
+affine group quantizer, the fused SwiGLU module and the per-layer error report,
+``native.py:88-264``) are alternative engines, not part of the EXL3 path.
 """
 
 from __future__ import annotations
-
-from dataclasses import dataclass
 
 import torch
 
 from . import ops
 from .layer import EXL3Layer
-from .linear import EXL3Linear, layer_runtime
+from .linear import layer_runtime
 
 # One stripe of output columns at a time (multiple of 128), native.py:45.
 PUBLIC_CHUNK_COLS = 8192
@@ -62,76 +61,3 @@ def folded_linear_from_exl3(layer: EXL3Layer, *, device="cuda") -> torch.nn.Line
             lin.bias.copy_(torch.from_numpy(layer.bias).to(torch.float16))
     lin.requires_grad_(False)
     return lin
-
-
-class FusedSwiGLU(torch.nn.Module):
-    """gate_proj + up_proj folded into one matmul (``FusedSwiGLU``, native.py:127-139)."""
-
-    def __init__(self, gate_up: torch.nn.Module, down: torch.nn.Module) -> None:
-        super().__init__()
-        self.gate_up = gate_up
-        self.down = down
-
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
-        g, u = self.gate_up(x).chunk(2, dim=-1)
-        return self.down(torch.nn.functional.silu(g) * u)
-
-
-def _fuse_two_linears(a: torch.nn.Linear, b: torch.nn.Linear) -> torch.nn.Linear:
-    out = torch.nn.Linear(a.in_features, a.out_features + b.out_features, bias=False,
-                          device=a.weight.device, dtype=a.weight.dtype)
-    with torch.no_grad():
-        out.weight.copy_(torch.cat([a.weight, b.weight], dim=0))
-    out.requires_grad_(False)
-    return out
-
-
-def fuse_mlps(model) -> int:
-    """Replace folded bias-free gate/up/down MLPs (``model.layers[i].mlp``) by
-    :class:`FusedSwiGLU` (``fuse_mlps``, native.py:166-185). Exact."""
-    n = 0
-    for layer in model.layers:
-        mlp = getattr(layer, "mlp", None)
-        gate = getattr(mlp, "gate_proj", None)
-        up = getattr(mlp, "up_proj", None)
-        down = getattr(mlp, "down_proj", None)
-        if gate is None or up is None or down is None:
-            continue
-        if not (type(gate) is torch.nn.Linear and type(up) is torch.nn.Linear):
-            continue
-        if gate.bias is not None or up.bias is not None:
-            continue
-        layer.mlp = FusedSwiGLU(_fuse_two_linears(gate, up), down)
-        n += 1
-    return n
-
-
-@dataclass
-class LayerError:
-    """Output-space error of a converted layer vs the exact EXL3 path (native.py:188-201)."""
-
-    key: str
-    engine: str
-    rms_ref: float
-    rms_err: float
-
-    @property
-    def rel(self) -> float:
-        return self.rms_err / self.rms_ref if self.rms_ref else 0.0
-
-    def __str__(self) -> str:
-        return f"{self.key}: rel RMS err {self.rel:.2e} ({self.engine})"
-
-
-def layer_error(layer: EXL3Layer, module: torch.nn.Module, engine: str, *, rows: int = 8,
-                device="cuda") -> LayerError:
-    """RMS error of ``module`` against ``EXL3Linear(layer)`` on ``rows`` seeded
-    N(0, 0.5^2) activations (``layer_error``, native.py:204-214)."""
-    gen = torch.Generator(device="cpu").manual_seed(0)
-    x = (torch.randn((rows, layer.in_features), generator=gen) * 0.5).to(torch.float16).to(device)
-    with torch.no_grad():
-        y_ref = EXL3Linear(layer, device=device)(x).float()
-        y_new = module(x).float()
-    rms_ref = float(torch.sqrt(torch.mean(y_ref * y_ref)))
-    rms_err = float(torch.sqrt(torch.mean((y_new - y_ref) ** 2)))
-    return LayerError(key=layer.key, engine=engine, rms_ref=rms_ref, rms_err=rms_err)

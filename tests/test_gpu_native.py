@@ -48,48 +48,9 @@ def test_folded_linear_tracks_exact_layer(cuda, oracle, bias):
     lin = native.folded_linear_from_exl3(layer, device=cuda)
     assert isinstance(lin, torch.nn.Linear) and lin.weight.dtype == torch.float16
     assert tuple(lin.weight.shape) == (384, 512) and (lin.bias is not None) == bias
-    err = native.layer_error(layer, lin, "fold16", device=cuda)
-    assert err.key == layer.key and err.engine == "fold16"
-    assert err.rel < 2e-3, str(err)
     rng = np.random.default_rng(3)
     x = rng.standard_normal((5, 512)).astype(np.float16)
     y = lin(torch.from_numpy(x).to(cuda)).cpu().numpy()
     ref = oracle.linear_forward(layer.trellis, 4, int(layer.codebook_mode), layer.suh, layer.svh, x,
                                 bias=layer.bias)
     assert rel_l2(y, ref) < 2e-3
-
-
-def test_fuse_mlps_is_exact(cuda):
-    from ponyexl3_amd import make_exl3_layer, native
-
-    class MLP(torch.nn.Module):
-        def __init__(self, g, u, d):
-            super().__init__()
-            self.gate_proj, self.up_proj, self.down_proj = g, u, d
-
-        def forward(self, x):
-            return self.down_proj(torch.nn.functional.silu(self.gate_proj(x)) * self.up_proj(x))
-
-    class Block(torch.nn.Module):
-        def __init__(self, mlp):
-            super().__init__()
-            self.mlp = mlp
-
-    class Model(torch.nn.Module):
-        def __init__(self, blocks):
-            super().__init__()
-            self.layers = torch.nn.ModuleList(blocks)
-
-    def fold(seed, n_in, n_out):
-        return native.folded_linear_from_exl3(
-            make_exl3_layer(k=4, in_features=n_in, out_features=n_out, seed=seed), device=cuda)
-
-    model = Model([Block(MLP(fold(1, 128, 256), fold(2, 128, 256), fold(3, 256, 128))),
-                   Block(torch.nn.Identity())])
-    x = torch.randn((3, 128), device=cuda).half() * 0.1
-    with torch.no_grad():
-        before = model.layers[0].mlp(x)
-        assert native.fuse_mlps(model) == 1
-        assert isinstance(model.layers[0].mlp, native.FusedSwiGLU)
-        after = model.layers[0].mlp(x)
-    assert float((before.float() - after.float()).abs().max()) <= 2e-3 * float(before.float().abs().max())

@@ -113,3 +113,39 @@ def test_errors(tmp_path):
         loader.layer_meta_from_config(d, "model.layers.9.mlp.gate_proj")
     with pytest.raises(FileNotFoundError):
         loader.list_exl3_layers(os.path.join(d, "nowhere"))
+
+
+def test_directory_is_scanned_once_and_shards_found_without_an_index(tmp_path):
+    """No index file and shards in a sub-directory: the tensor table comes from the
+    shard headers, every shard is parsed once however many tensors are read, and the
+    meta record is the package's own type (attribute and item access)."""
+    layers = _layers()
+    d = _write_checkpoint(tmp_path, layers, shards=2)
+    os.remove(os.path.join(d, "model.safetensors.index.json"))
+    sub = tmp_path / "shards"
+    sub.mkdir()
+    for fn in os.listdir(d):
+        if fn.endswith(".safetensors"):
+            os.rename(os.path.join(d, fn), str(sub / fn))
+    loader.clear_weight_index_cache(d)
+    opened = []
+    orig = loader._Shard.__init__
+
+    def counting(self, path):
+        opened.append(path)
+        orig(self, path)
+
+    loader._Shard.__init__ = counting
+    try:
+        got = loader.load_all_exl3_layers(d)
+        loader.load_exl3_layer(d, "lm_head")
+    finally:
+        loader._Shard.__init__ = orig
+    assert sorted(os.path.basename(p) for p in opened) == ["model-00000.safetensors", "model-00001.safetensors"]
+    for l in layers:
+        np.testing.assert_array_equal(got[l.key].trellis, l.trellis)
+    meta = loader.layer_meta_from_config(d, "lm_head")
+    assert isinstance(meta, loader.LayerMeta) and meta.k == meta["k"] == 6
+    assert meta.as_dict()["trellis_shape"] == (8, 8, 96)
+    ck = loader.open_checkpoint(d)
+    assert ck is loader.open_checkpoint(d) and ck.tensor("no.such.tensor") is None
