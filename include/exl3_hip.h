@@ -121,11 +121,16 @@ int exl3_had128_pre(const uint16_t *x, int rows, int n, const uint16_t *suh, int
  *              ponyexl3/mlx/exl3_moe.py:122-136, with the unsort of :768)
  *   i = in_index, s = scale_index, o = out_index: device int32[rows], or NULL for
  *   the identity; scale rows are scale_ld elements apart (a multiple of 8).
+ * x has n_in_rows rows, scale n_scale_rows, out n_out_rows: a table entry outside its
+ * range (negative included) makes the kernel skip that row - nothing is read or
+ * written for it - and with a NULL table `rows` must not exceed the buffer's rows
+ * (EXL3_E_BAD_SHAPE).
  * x, out fp16 rows of n elements (n a multiple of 128); x, scale, out 16-byte aligned.
  */
-int exl3_had128_rows(const uint16_t *x, int rows, int n, const int32_t *in_index,
-                     const uint16_t *scale, const int32_t *scale_index, size_t scale_ld, int post,
-                     uint16_t *out, const int32_t *out_index, void *stream);
+int exl3_had128_rows(const uint16_t *x, int n_in_rows, int rows, int n, const int32_t *in_index,
+                     const uint16_t *scale, int n_scale_rows, const int32_t *scale_index,
+                     size_t scale_ld, int post, uint16_t *out, int n_out_rows,
+                     const int32_t *out_index, void *stream);
 
 /*
  * Output-side Hadamard-128: optional split-K reduction, the fp16 cast of the
@@ -220,6 +225,9 @@ int exl3_gemm(const uint16_t *xh, int rows, size_t ldx, const uint16_t *trellis,
  *              reference builds the same table on the device and sizes it for
  *              the worst case, ponyexl3/mlx/exl3_moe.py:79-98, 722-723)
  *   y_out      fp16 [n_rows][ldy] (ldy >= 16*group_tiles), same row order as xh
+ * The table comes from device memory and is checked by the kernel: an entry whose
+ * group is outside [0, n_groups) or whose first row is negative is skipped, and its
+ * end row is clamped to n_rows.
  */
 int exl3_gemm_grouped(const uint16_t *xh, int n_rows, size_t ldx, const uint16_t *trellis,
                       int in_tiles, int out_tiles, int K, int cb, int tn_base, int group_tiles,

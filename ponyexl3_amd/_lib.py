@@ -57,7 +57,7 @@ PROTOTYPES = {
     "exl3_gemm": (_i, [_vp, _i, _sz, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp, _sz, _vp]),
     "exl3_gemm_workspace_bytes": (_sz, [_i, _i, _i]),
     "exl3_gemm_grouped": (_i, [_vp, _i, _sz, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _i, _vp, _sz, _vp]),
-    "exl3_had128_rows": (_i, [_vp, _i, _i, _vp, _vp, _vp, _sz, _i, _vp, _vp, _vp]),
+    "exl3_had128_rows": (_i, [_vp, _i, _i, _i, _vp, _vp, _i, _vp, _sz, _i, _vp, _i, _vp, _vp]),
     "exl3_linear_forward": (
         _i,
         [_vp, _i, _vp, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _sz, _vp],

@@ -141,9 +141,10 @@ int launch_gemm_grouped(const uint16_t* xh, int n_rows, size_t ldx, const uint16
                         int n_groups, const int32_t* group_tab, int n_row_blocks, int block_rows,
                         uint16_t* y_out, size_t ldy, hipStream_t stream);
 
-int launch_had_rows(const uint16_t* x, int rows, int n, const int32_t* in_index,
-                    const uint16_t* scale, const int32_t* scale_index, size_t scale_ld, int post,
-                    uint16_t* out, const int32_t* out_index, hipStream_t stream);
+int launch_had_rows(const uint16_t* x, int n_in_rows, int rows, int n, const int32_t* in_index,
+                    const uint16_t* scale, int n_scale_rows, const int32_t* scale_index,
+                    size_t scale_ld, int post, uint16_t* out, int n_out_rows,
+                    const int32_t* out_index, hipStream_t stream);
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 

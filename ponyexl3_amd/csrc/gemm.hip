@@ -101,7 +101,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
     const uint32_t* __restrict__ trellis, const half_t* __restrict__ xh, half_t* __restrict__ y,
     float* __restrict__ partial, int rows_arg, size_t ldx, size_t ldy, int in_tiles, int out_tiles,
     int tn_offset_arg, int tn_count_arg, int n_row_blocks, int full_tiles, int split,
-    int ksteps_per_split, const int4* __restrict__ group_tab, int group_tiles,
+    int ksteps_per_split, const int4* __restrict__ group_tab, int group_tiles, int n_groups,
     const int* __restrict__ block_sub, size_t sub_stride) {
     extern __shared__ __attribute__((aligned(16))) half_t smem[];
     constexpr int BM = 32 * MI;
@@ -120,8 +120,11 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
     int g, m0, rows, tn_offset, tn_count;
     if (group_tab) {
         const int n_col_blocks = (group_tiles + 15) >> 4;
-        const int4 t = group_tab[blockIdx.x / n_col_blocks];
-        if (t.y >= t.z) return;  // whole workgroup, before any barrier
+        int4 t = group_tab[blockIdx.x / n_col_blocks];
+        // the table is caller memory: a group outside the trellis slice or a row range
+        // outside xh / y would fault, so such entries are dropped / clamped
+        if (t.z > rows_arg) t.z = rows_arg;
+        if (t.x < 0 || t.x >= n_groups || t.y < 0 || t.y >= t.z) return;  // whole workgroup, before any barrier
         work.tile = 0;
         work.k_begin = 0;
         work.k_end = in_tiles / 4;
@@ -533,8 +536,8 @@ static int launch_gemm_mi(const GemmPlan& p, const uint16_t* xh, int rows, size_
     gemm_kernel<K, CB, MI><<<dim3(units), dim3(kGemmThreads), lds, stream>>>(
         reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<const half_t*>(xh),
         reinterpret_cast<half_t*>(y_out), partial, rows, ldx, ldy, in_tiles, out_tiles, tn_offset,
-        tn_count, p.n_row_blocks, p.full_tiles, p.split, p.ksteps_per_split, nullptr, 0, block_sub,
-        sub_stride);
+        tn_count, p.n_row_blocks, p.full_tiles, p.split, p.ksteps_per_split, nullptr, 0, 0,
+        block_sub, sub_stride);
     if (int rc = launch_status()) return rc;
     if (post) {  // only passed when every tile is split
         gemm_fixup_post_kernel<MI><<<dim3((unsigned)p.split_tiles, 4 * MI), dim3(256), 0, stream>>>(
@@ -599,9 +602,9 @@ int launch_gemm(const uint16_t* xh, int rows, size_t ldx, const uint16_t* trelli
 template <int K, int CB, int MI>
 static int launch_gemm_grouped_mi(const uint16_t* xh, int n_rows, size_t ldx,
                                   const uint16_t* trellis, int in_tiles, int out_tiles,
-                                  int tn_base, int group_tiles, const int32_t* group_tab,
-                                  int n_row_blocks, uint16_t* y_out, size_t ldy,
-                                  hipStream_t stream) {
+                                  int tn_base, int group_tiles, int n_groups,
+                                  const int32_t* group_tab, int n_row_blocks, uint16_t* y_out,
+                                  size_t ldy, hipStream_t stream) {
     constexpr size_t lds = (2 * (size_t)(32 * MI) * 64 + 2 * (size_t)kGemmStageB) * sizeof(half_t);
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_kernel<K, CB, MI>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -612,7 +615,7 @@ static int launch_gemm_grouped_mi(const uint16_t* xh, int n_rows, size_t ldx,
         reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<const half_t*>(xh),
         reinterpret_cast<half_t*>(y_out), nullptr, n_rows, ldx, ldy, in_tiles, out_tiles, tn_base,
         group_tiles, 1, 0, 1, in_tiles / 4, reinterpret_cast<const int4*>(group_tab), group_tiles,
-        nullptr, 0);
+        n_groups, nullptr, 0);
     return launch_status();
 }
 
@@ -636,17 +639,17 @@ int launch_gemm_grouped(const uint16_t* xh, int n_rows, size_t ldx, const uint16
         if (block_rows == 64)
             return launch_gemm_grouped_mi<k.value, c.value, 2>(xh, n_rows, ldx, trellis, in_tiles,
                                                                out_tiles, tn_base, group_tiles,
-                                                               group_tab, n_row_blocks, y_out, ldy,
-                                                               stream);
+                                                               n_groups, group_tab, n_row_blocks,
+                                                               y_out, ldy, stream);
         if (block_rows == 128)
             return launch_gemm_grouped_mi<k.value, c.value, 4>(xh, n_rows, ldx, trellis, in_tiles,
                                                                out_tiles, tn_base, group_tiles,
-                                                               group_tab, n_row_blocks, y_out, ldy,
-                                                               stream);
+                                                               n_groups, group_tab, n_row_blocks,
+                                                               y_out, ldy, stream);
         return launch_gemm_grouped_mi<k.value, c.value, 8>(xh, n_rows, ldx, trellis, in_tiles,
                                                            out_tiles, tn_base, group_tiles,
-                                                           group_tab, n_row_blocks, y_out, ldy,
-                                                           stream);
+                                                           n_groups, group_tab, n_row_blocks, y_out,
+                                                           ldy, stream);
     });
 }
 

@@ -40,16 +40,25 @@ __device__ __forceinline__ void wht128(float& a, float& b, int lane) {
 
 // Optional row gathers / scatter of the wide kernels: kernel row r reads input row
 // in_index[r], scale vector scale_index[r] (scale_ld elements apart) and writes
-// output row out_index[r]; a NULL table is the identity.
+// output row out_index[r]; a NULL table is the identity. The tables come from the
+// caller's memory: a row whose input, scale or output index falls outside
+// [0, n_in) / [0, n_scale) / [0, n_out) is skipped (nothing is read or written for it).
 struct RowMap {
     int per_row;
     const int32_t* in_index;
     const int32_t* scale_index;
     const int32_t* out_index;
     size_t scale_ld;
+    unsigned n_in, n_scale, n_out;  // rows behind x, scale and out (per_row mode only)
     __device__ size_t in_row(size_t r) const { return in_index ? (size_t)in_index[r] : r; }
     __device__ size_t scale_row(size_t r) const { return scale_index ? (size_t)scale_index[r] : r; }
     __device__ size_t out_row(size_t r) const { return out_index ? (size_t)out_index[r] : r; }
+    __device__ bool row_ok(size_t r, bool uses_scale) const {
+        if (!per_row) return true;
+        // negative entries wrap to huge unsigned values and fail the same test
+        return in_row(r) < (size_t)n_in && out_row(r) < (size_t)n_out &&
+               (!uses_scale || scale_row(r) < (size_t)n_scale);
+    }
 };
 
 // v[j] = element 8*(lane & 15) + j of the lane group's block, unnormalised WHT in place.
@@ -97,6 +106,7 @@ __global__ __launch_bounds__(256) void had_pre_wide_kernel(const half_t* __restr
                                                            int n_sub, RowMap map) {
     const int lane = threadIdx.x & 63;
     const size_t rs = blockIdx.x;
+    if (!map.row_ok(rs, suh != nullptr)) return;
     // source row and scale vector: (row, sub) product for stacked siblings, or
     // per-row tables for rows that were sorted by expert
     const half_t* xr = x + (map.per_row ? map.in_row(rs) : rs / n_sub) * (size_t)n;
@@ -132,6 +142,7 @@ __global__ __launch_bounds__(256) void had_post_wide_kernel(const half_t* __rest
                                                             half_t* out, int n, RowMap map) {
     const int lane = threadIdx.x & 63;
     const size_t rs = blockIdx.x;
+    if (!map.row_ok(rs, svh != nullptr)) return;
     if (svh && map.per_row) svh += map.scale_row(rs) * map.scale_ld;
     const half_t* yr = y + map.in_row(rs) * (size_t)n;
     half_t* orow = out + map.out_row(rs) * (size_t)n;
@@ -322,14 +333,22 @@ int launch_had_post(const void* y, int y_is_fp32, int n_sum, size_t sum_stride, 
 }
 
 // Per-row scale vectors (rows that belong to different experts): wide kernels only.
-int launch_had_rows(const uint16_t* x, int rows, int n, const int32_t* in_index,
-                    const uint16_t* scale, const int32_t* scale_index, size_t scale_ld, int post,
-                    uint16_t* out, const int32_t* out_index, hipStream_t stream) {
+int launch_had_rows(const uint16_t* x, int n_in_rows, int rows, int n, const int32_t* in_index,
+                    const uint16_t* scale, int n_scale_rows, const int32_t* scale_index,
+                    size_t scale_ld, int post, uint16_t* out, int n_out_rows,
+                    const int32_t* out_index, hipStream_t stream) {
     if (!x || !out || !scale) return EXL3_E_NULL_POINTER;
-    if (rows < 0 || n <= 0 || n % 128 || scale_ld % 8) return EXL3_E_BAD_SHAPE;
+    if (rows < 0 || n <= 0 || n % 128 || scale_ld % 8 || n_in_rows < 0 || n_scale_rows < 0 ||
+        n_out_rows < 0)
+        return EXL3_E_BAD_SHAPE;
+    // identity maps must stay inside their buffers as well
+    if ((!in_index && rows > n_in_rows) || (!scale_index && rows > n_scale_rows) ||
+        (!out_index && rows > n_out_rows))
+        return EXL3_E_BAD_SHAPE;
     if (!aligned16(x) || !aligned16(out) || !aligned16(scale)) return EXL3_E_BAD_SHAPE;
     if (rows == 0) return EXL3_OK;
-    const RowMap map{1, in_index, scale_index, out_index, scale_ld};
+    const RowMap map{1, in_index, scale_index, out_index, scale_ld, (unsigned)n_in_rows,
+                     (unsigned)n_scale_rows, (unsigned)n_out_rows};
     if (post)
         had_post_wide_kernel<<<dim3((unsigned)rows, wide_row_parts(rows, n)), dim3(256), 0, stream>>>(
             reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(scale), nullptr,
@@ -343,12 +362,14 @@ int launch_had_rows(const uint16_t* x, int rows, int n, const int32_t* in_index,
 
 }  // namespace exl3
 
-EXL3_EXPORT int exl3_had128_rows(const uint16_t* x, int rows, int n, const int32_t* in_index,
-                                 const uint16_t* scale, const int32_t* scale_index,
-                                 size_t scale_ld, int post, uint16_t* out,
-                                 const int32_t* out_index, void* stream) {
-    return exl3::launch_had_rows(x, rows, n, in_index, scale, scale_index, scale_ld, post, out,
-                                 out_index, exl3::as_stream(stream));
+EXL3_EXPORT int exl3_had128_rows(const uint16_t* x, int n_in_rows, int rows, int n,
+                                 const int32_t* in_index, const uint16_t* scale, int n_scale_rows,
+                                 const int32_t* scale_index, size_t scale_ld, int post,
+                                 uint16_t* out, int n_out_rows, const int32_t* out_index,
+                                 void* stream) {
+    return exl3::launch_had_rows(x, n_in_rows, rows, n, in_index, scale, n_scale_rows, scale_index,
+                                 scale_ld, post, out, n_out_rows, out_index,
+                                 exl3::as_stream(stream));
 }
 
 EXL3_EXPORT int exl3_had128_pre(const uint16_t* x, int rows, int n, const uint16_t* suh, int n_sub,

@@ -10,6 +10,8 @@ Hadamard block never straddles two members).
 
 from __future__ import annotations
 
+import weakref
+
 import numpy as np
 import torch
 
@@ -61,8 +63,9 @@ class FusedEXL3Group(torch.nn.Module):
         # member of every 256-column block, for the one-launch prefill GEMM
         self._block_sub = (self._group_sub[::2].contiguous()
                            if all(n % 256 == 0 for n in self._out_features) else None)
-        self._cache_x = None
+        self._cache_key = None
         self._cache_out = None
+        self._cache_served: set = set()
 
     def extra_repr(self) -> str:
         return f"members={self._keys}, k={self._k}"
@@ -77,11 +80,35 @@ class FusedEXL3Group(torch.nn.Module):
         outs = torch.split(y, self._out_features, dim=-1)
         return tuple(o.reshape(lead + (n,)) for o, n in zip(outs, self._out_features))
 
-    def cached(self, x: torch.Tensor) -> tuple[torch.Tensor, ...]:
-        if self._cache_out is None or self._cache_x is not x:
+    def _same_input(self, x: torch.Tensor) -> bool:
+        """Whether x is the input the cached outputs were computed from. The reference
+        compares object identity (ponyexl3/mlx/exl3_fused.py:204-208), which is enough
+        for immutable mlx arrays. A torch tensor can be refilled in place (static
+        decode buffers, HIP-graph inputs), so the version counter must match too; the
+        tensor is held weakly (a freed tensor's address can be handed out again); and a
+        result computed eagerly must not stand in for a launch that a graph capture
+        has to record."""
+        if self._cache_out is None or self._cache_key is None:
+            return False
+        ref, version, capturing = self._cache_key
+        return (ref() is x and version == x._version
+                and capturing == (x.is_cuda and torch.cuda.is_current_stream_capturing()))
+
+    def cached(self, x: torch.Tensor, idx: int | None = None) -> tuple[torch.Tensor, ...]:
+        """Outputs of all members for x, computed once per distinct input and dropped
+        as soon as every member has been served (nothing is kept alive after that)."""
+        if not self._same_input(x):
             self._cache_out = self.forward_all(x)
-            self._cache_x = x
-        return self._cache_out
+            self._cache_key = (weakref.ref(x), x._version,
+                               x.is_cuda and torch.cuda.is_current_stream_capturing())
+            self._cache_served = set()
+        outs = self._cache_out
+        if idx is not None:
+            self._cache_served.add(idx)
+            if len(self._cache_served) == len(self._out_features):
+                self._cache_out = None
+                self._cache_key = None
+        return outs
 
     def sibling(self, idx: int) -> "FusedEXL3Sibling":
         return FusedEXL3Sibling(self, idx)
@@ -103,4 +130,4 @@ class FusedEXL3Sibling(torch.nn.Module):
         return f"{self._group._keys[self._idx]} (member {self._idx})"
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return self._group.cached(x)[self._idx]
+        return self._group.cached(x, self._idx)[self._idx]

@@ -450,8 +450,9 @@ def had128_rows(x2d: torch.Tensor, scale: torch.Tensor, post: bool, *, rows: int
         raise ValueError(f"feature dim {n} not divisible by 128")
     out = torch.empty((rows, n), dtype=torch.float16, device=x2d.device)
     rc = _lib.load().exl3_had128_rows(
-        _ptr(x2d), rows, n, _ptr(in_index), _ptr(scale), _ptr(scale_index), scale.stride(0),
-        int(bool(post)), _ptr(out), _ptr(out_index), _stream())
+        _ptr(x2d), x2d.shape[0], rows, n, _ptr(in_index), _ptr(scale), scale.shape[0],
+        _ptr(scale_index), scale.stride(0), int(bool(post)), _ptr(out), rows, _ptr(out_index),
+        _stream())
     _lib.check(rc, "exl3_had128_rows")
     return out
 

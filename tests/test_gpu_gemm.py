@@ -1,5 +1,7 @@
 """MFMA prefill GEMM against the oracle-decoded fp16 weights times xh
 (fp32 accumulation, rel-L2 <= 1e-3)."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -90,9 +92,9 @@ def test_small_batch_and_prefill_kernels_agree(cuda):
 
 
 def test_config3_prefill_against_decoded_weights(cuda, oracle):
-    """M = 2048 on the q_proj shape 5120 -> 8192: compare with oracle-checked
-    decoded fp16 weights times xh in fp32 (decode_full is bit-exact, see
-    test_gpu_decode.py; a column block is checked against the oracle here)."""
+    """M = 2048 on the q_proj shape 5120 -> 8192: compare with the decoded fp16
+    weights times xh in fp32; the decoded matrix (all 41.9 M weights) is first
+    checked bit for bit against the oracle's decode."""
     from ponyexl3_amd import ops
 
     rng = np.random.default_rng(30_004)
@@ -102,9 +104,8 @@ def test_config3_prefill_against_decoded_weights(cuda, oracle):
     xh = torch.randn((2048, 5120), generator=g).to(torch.float16).to(cuda)
     y = ops.inner_gemm(xh, tr, 4, 0)
     w = ops.decode_full(tr, 4, 0)
-    np.testing.assert_array_equal(
-        w[:, 1024:1152].cpu().numpy().view(np.uint16),
-        oracle.decode_trellis(tr_np, 4, 0, tn_offset=64, tn_count=8).view(np.uint16))
+    np.testing.assert_array_equal(w.cpu().numpy().view(np.uint16),
+                                  oracle.decode_trellis(tr_np, 4, 0).view(np.uint16))
     ref = xh.float() @ w.float()
     err = (y.float() - ref).norm() / ref.norm()
     assert float(err) < 5e-4
@@ -162,6 +163,41 @@ def test_config3_split_shapes_against_decoded_weights(cuda, n_in, n_out):
         err = (y[:, c0:c0 + 8192].float() - ref).norm() / ref.norm()
         worst = max(worst, float(err))
     assert worst < 5e-4
+
+
+def test_grouped_gemm_drops_bad_table_entries(cuda, oracle):
+    """The row-block table of exl3_gemm_grouped is caller memory: entries that name a
+    group outside the stack, a negative first row or an end row past the activations
+    must not make the kernel read or write out of bounds. Bad entries are skipped,
+    an end row past n_rows is clamped; the valid blocks come out as usual."""
+    from ponyexl3_amd import ops
+
+    rng = np.random.default_rng(77)
+    n_groups, gt = 3, 16  # three groups of 256 columns each
+    tr_np = rng.integers(0, 65536, size=(16, n_groups * gt, 64), dtype=np.uint16)  # in = 256
+    tr = ops.as_trellis_tensor(tr_np, cuda)
+    xh_np = rng.standard_normal((96, 256)).astype(np.float16)
+    xh = _t(xh_np, cuda)
+    table = torch.tensor([[0, 0, 40, 0],      # group 0: rows 0..39
+                          [7, 40, 60, 0],     # group out of range: skipped
+                          [1, -5, 20, 0],     # negative first row: skipped
+                          [2, 64, 4000, 0],   # end row past the matrix: clamped to 96
+                          [-1, 0, 10, 0]],    # negative group: skipped
+                         dtype=torch.int32, device=cuda)
+    sentinel = 12345.0
+    y = torch.full((96, gt * 16), sentinel, dtype=torch.float16, device=cuda)
+    from ponyexl3_amd import _lib
+    rc = _lib.load().exl3_gemm_grouped(
+        ctypes.c_void_p(xh.data_ptr()), 96, 256, ctypes.c_void_p(tr.data_ptr()), 16, n_groups * gt, 4, 0,
+        0, gt, n_groups, ctypes.c_void_p(table.data_ptr()), table.shape[0], 64,
+        ctypes.c_void_p(y.data_ptr()), gt * 16, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    w = oracle.decode_trellis(tr_np, 4, 0).astype(np.float64)
+    got = y.cpu().numpy()
+    assert rel_l2(got[:40], xh_np[:40].astype(np.float64) @ w[:, :256]) < 5e-4
+    assert rel_l2(got[64:96], xh_np[64:96].astype(np.float64) @ w[:, 512:768]) < 5e-4
+    assert (got[40:64] == np.float16(sentinel)).all()  # rows of the dropped entries are untouched
 
 
 def test_errors(cuda):

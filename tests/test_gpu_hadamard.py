@@ -96,6 +96,41 @@ def test_involution_at_scale(cuda):
     assert float(((nx - ny).abs() / nx).max()) < TOL
 
 
+def test_row_tables_out_of_range_are_skipped(cuda, oracle):
+    """exl3_had128_rows takes its gather / scatter tables from caller memory: an entry
+    outside the buffer it indexes (negative included) makes the kernel skip that row;
+    the other rows come out as usual and nothing outside the buffers is touched."""
+    import ctypes
+
+    from ponyexl3_amd import _lib
+
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((6, 256)).astype(np.float16)
+    scale = np.where(rng.random((3, 256)) > 0.5, -1.0, 1.0).astype(np.float16)
+    in_index = np.array([0, 5, 6, -1, 2, 3], dtype=np.int32)       # 6 and -1 are out of range
+    scale_index = np.array([0, 1, 2, 0, 3, 2], dtype=np.int32)     # 3 is out of range
+    out_index = np.array([0, 1, 2, 3, 4, 9], dtype=np.int32)       # 9 is out of range
+    xt, st = torch.from_numpy(x).to(cuda), torch.from_numpy(scale).to(cuda)
+    ii, si, oi = (torch.from_numpy(a).to(cuda) for a in (in_index, scale_index, out_index))
+    out = torch.full((6, 256), 777.0, dtype=torch.float16, device=cuda)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    lib = _lib.load()
+    rc = lib.exl3_had128_rows(p(xt), 6, 6, 256, p(ii), p(st), 3, p(si), 256, 0, p(out), 6, p(oi),
+                              ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    for r in (0, 1):  # the two rows whose three indices are all valid
+        want = oracle.had_r_128(x[in_index[r]][None].astype(np.float32),
+                                pre_scale=scale[scale_index[r]]).astype(np.float16)[0]
+        np.testing.assert_array_equal(got[out_index[r]], want)
+    assert (got[2:] == np.float16(777.0)).all()
+    # identity maps longer than their buffers are refused on the host
+    rc = lib.exl3_had128_rows(p(xt), 4, 6, 256, None, p(st), 3, p(si), 256, 0, p(out), 6, None,
+                              ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == _lib.EXL3_E_BAD_SHAPE
+
+
 def test_errors(cuda):
     from ponyexl3_amd import ops
 

@@ -218,6 +218,25 @@ def test_single_slot_cache_computes_once(cuda):
     assert s0.out_features == 128 and s0.in_features == 256
 
 
+def test_sibling_cache_sees_in_place_updates(cuda):
+    """A static input buffer refilled in place between two decode steps must not be
+    served the previous step's outputs, and the cache holds nothing once every
+    member has read it."""
+    from ponyexl3_amd import EXL3Linear, FusedEXL3Group, make_exl3_layer
+
+    layers = [make_exl3_layer(k=4, in_features=256, out_features=128, seed=90 + i, key=f"v{i}") for i in range(2)]
+    group = FusedEXL3Group(layers)
+    s0, s1 = group.sibling(0), group.sibling(1)
+    x = torch.randn((1, 256), device=cuda).half()
+    a0 = s0(x).clone()
+    x.copy_(torch.randn((1, 256), device=cuda).half())  # same tensor object, new values
+    b1 = s1(x)
+    assert torch.equal(b1, EXL3Linear(layers[1])(x))
+    b0 = s0(x)
+    assert torch.equal(b0, EXL3Linear(layers[0])(x)) and not torch.equal(a0, b0)
+    assert group._cache_out is None and group._cache_key is None  # both members served
+
+
 @pytest.mark.parametrize("rows", [1, 3, 8, 13, 16])
 @pytest.mark.parametrize("k,n_in,n_out", [(4, 512, 384), (3, 1024, 256), (6, 2176, 640), (4, 5120, 1024)])
 def test_one_launch_layer_equals_three_launch_chain(cuda, rows, k, n_in, n_out):
