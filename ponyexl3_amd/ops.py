@@ -40,11 +40,18 @@ def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
+def _buffer_key(device):
+    """Scratch buffers and counters belong to one (device, stream) pair: launches on
+    one stream are ordered, so they can share a buffer; two streams of a device
+    running EXL3 layers at the same time must not (the group counters and partial
+    rows of one launch would be read by the other)."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    return (device.type, index, torch.cuda.current_stream(index).cuda_stream)
+
+
 def workspace(device, nbytes: int) -> torch.Tensor:
-    """Per-device scratch buffer shared by all calls on that device (grown on
-    demand). Calls that overlap on different streams of one device would race
-    on it; the reference runs one stream too."""
-    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    """Scratch buffer of the current (device, stream), grown on demand."""
+    key = _buffer_key(device)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
         if buf is not None:
@@ -58,11 +65,12 @@ _gemm_workspaces: dict = {}
 
 
 def gemm_workspace(device, nbytes: int):
-    """Per-device scratch for the prefill GEMM's fp32 partial tiles (kept apart
-    from ``workspace``, which holds the GEMM's operands during a layer forward)."""
+    """Scratch of the current (device, stream) for the prefill GEMM's fp32 partial
+    tiles (kept apart from ``workspace``, which holds the GEMM's operands during a
+    layer forward)."""
     if nbytes <= 0:
         return None
-    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    key = _buffer_key(device)
     buf = _gemm_workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
         if buf is not None:
@@ -76,9 +84,10 @@ _counters: dict = {}
 
 
 def sync_counters(device, n: int) -> torch.Tensor:
-    """Per-device int32 array of group counters for the one-launch layer kernel.
-    Zeroed when created; the kernel leaves it zero, so it is reused as is."""
-    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    """int32 array of group counters of the current (device, stream) for the
+    one-launch layer kernel. Zeroed when created; the kernel leaves it zero, so it
+    is reused as is."""
+    key = _buffer_key(device)
     buf = _counters.get(key)
     if buf is None or buf.numel() < n:
         if buf is not None:

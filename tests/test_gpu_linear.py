@@ -377,3 +377,35 @@ def test_sibling_prefill_in_one_gemm_launch(cuda, oracle, rows):
     x2, xt2 = _x(rng, (rows, 512), cuda)
     for o, l in zip(odd.forward_all(xt2), odd_layers):
         assert rel_l2(o.cpu().numpy(), _oracle_forward(oracle, l, x2)) <= TOL
+
+
+def test_two_streams_do_not_share_scratch(cuda):
+    """Layers running on two streams of one device at the same time: partial rows and
+    group counters are per (device, stream), so both streams get the results they get
+    when run alone."""
+    from ponyexl3_amd import make_exl3_layer, ops
+
+    la = make_exl3_layer(k=4, in_features=2176, out_features=640, seed=501)
+    lb = make_exl3_layer(k=3, in_features=4096, out_features=384, seed=502)
+    dev_t = lambda l: (ops.as_trellis_tensor(l.trellis, cuda), torch.from_numpy(l.suh).to(cuda),
+                       torch.from_numpy(l.svh).to(cuda))
+    ta, tb = dev_t(la), dev_t(lb)
+    xa = torch.randn((2, 2176), device=cuda).half()
+    xb = torch.randn((1, 4096), device=cuda).half()
+    ref_a = ops.linear_forward(xa, ta[0], 4, 0, ta[1], ta[2])
+    ref_b = ops.linear_forward(xb, tb[0], 3, 0, tb[1], tb[2])
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    outs_a, outs_b = [], []
+    with torch.cuda.stream(s1):
+        ws1 = ops.workspace(cuda, 1).data_ptr()
+        for _ in range(50):
+            outs_a.append(ops.linear_forward(xa, ta[0], 4, 0, ta[1], ta[2]))
+    with torch.cuda.stream(s2):
+        ws2 = ops.workspace(cuda, 1).data_ptr()
+        for _ in range(50):
+            outs_b.append(ops.linear_forward(xb, tb[0], 3, 0, tb[1], tb[2]))
+    torch.cuda.synchronize()
+    assert ws1 != ws2
+    assert all(torch.equal(o, ref_a) for o in outs_a)
+    assert all(torch.equal(o, ref_b) for o in outs_b)
