@@ -32,9 +32,14 @@
  *   exl3o_linear_forward   pinned: reference forward outputs on small layers
  *                          (tolerance: the reference sums in BLAS order),
  *                          public-weight identity.
- *   exl3o_moe_expert       composition of pinned parts; the reference has no CPU
- *                          twin for the MoE chain (only Metal kernels), so the
- *                          chain as a whole is "parity unpinned" beyond that.
+ *   MoE expert chain       (moe_experts_forward / glu in exl3_oracle.py) composition
+ *                          of the pinned linear forward with the GLU. The reference
+ *                          has no CPU twin of the chain (only Metal kernels) and so
+ *                          no vectors; it is pinned by what the mathematics fixes:
+ *                          SiLU and tanh-GELU against their closed forms in float64,
+ *                          and the chain against dense public-weight products
+ *                          y = (act(x Wg) * (x Wu)) Wd per expert, with wrong expert,
+ *                          exchanged gate/up and missing activation as failing cases.
  *   exl3o_quantize_tile_exact
  *                          exact Viterbi over the bitshift trellis
  *                          (convert/reference_search.py). Pinned: states and
