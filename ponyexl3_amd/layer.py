@@ -94,6 +94,20 @@ class EXL3Layer:
             raise ValueError(f"trellis shape {got} != expected {expected}")
 
 
+def pack_trellis_tiles(symbols: np.ndarray, k: int) -> np.ndarray:
+    """K-bit symbols (..., 256) -> packed tiles (..., 16*K) uint16, the bit order of
+    ``pack_trellis_tile`` (ponyexl3/ref/trellis.py:13-49): symbol c fills stream bits
+    [c*K, (c+1)*K) most significant bit first, and stream bit b is bit 31 - b % 32 of
+    little-endian 32-bit word b // 32 of the tile."""
+    sym = np.asarray(symbols).astype(np.uint32) & ((1 << k) - 1)
+    lead = sym.shape[:-1]
+    shifts = np.arange(k - 1, -1, -1, dtype=np.uint32)
+    bits = ((sym[..., None] >> shifts) & 1).reshape(lead + (8 * k, 32))  # stream order, 32 per word
+    weights = (np.uint32(1) << np.arange(31, -1, -1, dtype=np.uint32))
+    words = (bits * weights).sum(axis=-1, dtype=np.uint64).astype("<u4")
+    return np.ascontiguousarray(words).view("<u2").reshape(lead + (16 * k,)).astype(np.uint16)
+
+
 def make_exl3_layer(
     *,
     k: int = 4,
@@ -106,22 +120,44 @@ def make_exl3_layer(
     mul1: bool = False,
     bias: bool = False,
     key: str = "synthetic.layer",
+    ref_compatible: bool = False,
 ) -> EXL3Layer:
-    """Seeded synthetic layer. Every uint16 fill is a legal bitstream, so the
-    trellis is raw random words (``numpy.random.default_rng(seed)``); signs are
-    ``where(rng.random(n) > 0.5, -1, 1)`` drawn after the trellis, suh first."""
+    """Seeded synthetic layer. Every uint16 fill is a legal bitstream, so by default
+    the trellis is raw random words (``numpy.random.default_rng(seed)``); signs are
+    ``where(rng.random(n) > 0.5, -1, 1)`` drawn after the trellis, suh first.
+
+    ``ref_compatible=True`` reproduces ``ponyexl3.ref.synthetic.make_exl3_layer``
+    (ponyexl3/ref/synthetic.py:13-82) bit for bit: tile (i, j) packs 256 symbols
+    ``integers(0, 2**16, 256, uint32) & (2**K - 1)`` drawn from its own generator
+    seeded ``seed*1000 + i*10 + j``; signs and bias come from a separate
+    ``default_rng(seed)``, suh first, then svh, then ``standard_normal(out)`` cast to
+    fp16 and scaled by 0.01 in fp16. One generator per tile makes it slow for large
+    layers (65 536 tiles at 4096 x 4096), which is why it is not the default."""
     rng = np.random.default_rng(seed)
-    trellis = rng.integers(
-        0, 65536, size=(in_features // 16, out_features // 16, 16 * k), dtype=np.uint16
-    )
+    in_tiles, out_tiles = in_features // 16, out_features // 16
+    if ref_compatible:
+        sym = np.empty((in_tiles, out_tiles, 256), dtype=np.uint32)
+        for i in range(in_tiles):
+            for j in range(out_tiles):
+                sym[i, j] = np.random.default_rng(seed * 1000 + i * 10 + j).integers(
+                    0, 2**16, size=256, dtype=np.uint32)
+        trellis = pack_trellis_tiles(sym, k)
+    else:
+        trellis = rng.integers(0, 65536, size=(in_tiles, out_tiles, 16 * k), dtype=np.uint16)
 
     def _signs(n):
         return np.where(rng.random(n) > 0.5, -1.0, 1.0).astype(np.float16)
 
     suh_arr = _signs(in_features) if isinstance(suh, str) else suh
     svh_arr = _signs(out_features) if isinstance(svh, str) else svh
-    bias_arr = (rng.standard_normal(out_features) * 0.01).astype(np.float16) if bias else None
+    if not bias:
+        bias_arr = None
+    elif ref_compatible:
+        bias_arr = rng.standard_normal(out_features).astype(np.float16) * np.float16(0.01)
+    else:
+        bias_arr = (rng.standard_normal(out_features) * 0.01).astype(np.float16)
     return EXL3Layer(
-        key=key, in_features=in_features, out_features=out_features, k=k, trellis=trellis,
+        key="test.layer" if ref_compatible and key == "synthetic.layer" else key,
+        in_features=in_features, out_features=out_features, k=k, trellis=trellis,
         suh=suh_arr, svh=svh_arr, bias=bias_arr, mcg=mcg, mul1=mul1,
     )

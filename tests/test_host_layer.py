@@ -96,3 +96,38 @@ def test_tensor_core_perm_closed_form(oracle):
     np.testing.assert_array_equal(perm, oracle.tensor_core_perm())
     assert sorted(perm.tolist()) == list(range(256))
     np.testing.assert_array_equal(perm[tensor_core_perm_inverse()], np.arange(256))
+
+
+def test_ref_compatible_synthetic_layers_match_the_reference_bit_for_bit():
+    """make_exl3_layer(ref_compatible=True) against the layers that the reference's own
+    make_exl3_layer produced for tests/golden/forwards.npz (seed = 40 + K + 10*cb,
+    128 -> 256): trellis words, both sign vectors and the bias."""
+    from conftest import golden
+    from ponyexl3_amd import make_exl3_layer
+
+    g = golden("forwards.npz")
+    cases = [(k, cb, False) for k in range(1, 9) for cb in (0, 1)] + [(4, 2, False), (4, 0, True)]
+    for k, cb, bias in cases:
+        tag = f"k{k}_cb{cb}" + ("_bias" if bias else "")
+        layer = make_exl3_layer(k=k, in_features=128, out_features=256, seed=40 + k + 10 * cb,
+                                mcg=cb == 1, mul1=cb == 2, bias=bias, ref_compatible=True)
+        assert layer.key == "test.layer"
+        np.testing.assert_array_equal(layer.trellis, g[tag + "_trellis"], err_msg=tag)
+        np.testing.assert_array_equal(layer.suh.view(np.uint16), g[tag + "_suh"], err_msg=tag)
+        np.testing.assert_array_equal(layer.svh.view(np.uint16), g[tag + "_svh"], err_msg=tag)
+        if bias:
+            np.testing.assert_array_equal(layer.bias.view(np.uint16), g[tag + "_bias"].view(np.uint16))
+    pub = make_exl3_layer(k=4, in_features=128, out_features=256, seed=77, ref_compatible=True)
+    np.testing.assert_array_equal(pub.trellis, g["pub_trellis"])
+    np.testing.assert_array_equal(pub.suh.view(np.uint16), g["pub_suh"])
+
+
+def test_pack_trellis_tiles_matches_the_oracle_packer(oracle):
+    from ponyexl3_amd.layer import pack_trellis_tiles
+
+    rng = np.random.default_rng(3)
+    for k in range(1, 9):
+        sym = rng.integers(0, 65536, size=(3, 2, 256), dtype=np.uint16)
+        got = pack_trellis_tiles(sym, k)
+        want = oracle.pack_trellis((sym & ((1 << k) - 1)).astype(np.uint16), k)
+        np.testing.assert_array_equal(got, want)
