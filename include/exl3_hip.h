@@ -248,17 +248,25 @@ size_t exl3_gemm_workspace_bytes(int rows, int in_tiles, int tn_count);
  *   group_sub int32 [out/128] or NULL (required when n_sub > 1)
  *   y        fp16 [rows][out]
  *   workspace at least exl3_linear_workspace_bytes(rows, in, out, n_sub)
- *   counters int32 [counters_len >= out/128] or NULL. With counters and
- *            rows <= exl3_gemv_max_rows() the whole layer is ONE kernel launch:
- *            the last wavefront to finish a 128-column group reduces the splits
- *            and applies the output transform. The array must be all zero on
- *            entry and is all zero again when the launch has finished, so a
- *            caller zeroes it once and reuses it (calls that overlap on one
- *            array race). Above that and up to exl3_linear_small_max_rows() rows
- *            the counters serve the medium-batch kernel in the same way (two
- *            launches: input rotation, then everything else). NULL selects the
- *            three-launch chain (exl3_had128_pre, exl3_gemv_partials,
- *            exl3_had128_post) resp. the prefill GEMM.
+ *   counters int32 [counters_len], 8-byte aligned, or NULL. With counters and
+ *            rows <= exl3_gemv_max_rows() the whole layer is ONE kernel launch;
+ *            counters_len >= 2*rows*out. The workgroups that share a 128-column
+ *            group combine their partial rows in one of two ways, chosen by the
+ *            size of the launch: 64-bit fixed-point accumulators in this array,
+ *            one per (row, output column), updated with returning atomics (the
+ *            total does not depend on the arrival order; the workgroup whose add
+ *            completes the group applies the output transform), or fp32 partial
+ *            rows in the workspace plus one counter per group in this array (the
+ *            workgroup that brings the counter to its final value adds the partial
+ *            rows in index order). Either way the array must be all zero on entry
+ *            and is all zero again when the launch has finished, so a caller
+ *            zeroes it once and reuses it (calls that overlap on one array race),
+ *            and results are run-to-run deterministic. Above that and up to
+ *            exl3_linear_small_max_rows() rows the array serves the medium-batch
+ *            kernel as group counters (counters_len >= out/128; two launches: input
+ *            rotation, then everything else). NULL selects the three-launch chain
+ *            (exl3_had128_pre, exl3_gemv_partials, exl3_had128_post) resp. the
+ *            prefill GEMM.
  */
 int exl3_linear_forward(const uint16_t *x, int rows, const uint16_t *trellis, int in_tiles,
                         int out_tiles, int K, int cb, const uint16_t *suh, int n_sub,
@@ -273,16 +281,18 @@ size_t exl3_linear_workspace_bytes(int rows, int in_features, int out_features, 
  * workspace: code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc. It has no counterpart in the reference. Same arguments and
  * results as exl3_linear_forward with counters (the one-launch kernel), minus
- * workspace and counters: the split-K partial rows and the group counters live in
- * a device array inside the library (exl3_linear_static_scratch_bytes() = 16 MiB of
- * partial rows plus 4096 counters; every GPU the library runs on holds its copy
- * until the process ends). No hipMalloc, hipFree or other allocating call is made.
+ * workspace and counters: the kernel's split-K state (fp32 partial rows and group
+ * counters, or 64-bit accumulators, whichever reduction the launch uses) lives in a
+ * device array inside the library: exl3_linear_static_scratch_bytes() = 16 MiB for
+ * the partial rows plus as much for the counters / accumulators; every GPU the
+ * library runs on holds its copy until the process ends. No hipMalloc, hipFree or
+ * other allocating call is made.
  *   rows <= exl3_gemv_max_rows(), otherwise EXL3_E_UNSUPPORTED;
- *   exl3_linear_static_need_bytes(rows, in, out) must not exceed the scratch size
- *   and out/128 must not exceed 4096, otherwise EXL3_E_STATIC_LIMIT (nothing is
- *   launched).
+ *   exl3_linear_static_need_bytes(rows, in, out) must not exceed the scratch size,
+ *   otherwise EXL3_E_STATIC_LIMIT (nothing is launched).
  * All calls on one GPU share that GPU's array: calls that overlap there (two
- * streams, two threads) race. The counters are zero whenever no call is running.
+ * streams, two threads) race. The counter half is all zero whenever no call is
+ * running.
  */
 size_t exl3_linear_static_scratch_bytes(void);
 size_t exl3_linear_static_need_bytes(int rows, int in_features, int out_features);

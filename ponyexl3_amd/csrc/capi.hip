@@ -92,8 +92,9 @@ EXL3_EXPORT int exl3_linear_forward(const uint16_t* x, int rows, const uint16_t*
         const GemvPlan plan = plan_gemv(rows, in_tiles, n_groups);
         float* partial = reinterpret_cast<float*>(second);
         if (counters) {
-            // one launch: rotation, GEMV, split reduction and output transform fused
-            if (counters_len < (size_t)n_groups) return EXL3_E_WORKSPACE;
+            // one launch: rotation, GEMV, split reduction and output transform fused;
+            // the counters array holds the 64-bit accumulators (two ints each)
+            if (counters_len < linear_small_counter_ints(rows, out_features)) return EXL3_E_WORKSPACE;
             return launch_linear_small(x, rows, trellis, in_tiles, out_tiles, K, cb, suh, n_sub,
                                        group_sub, svh, bias, y, partial, counters,
                                        plan_linear_small(rows, in_tiles, n_groups), s);
@@ -175,17 +176,17 @@ EXL3_EXPORT int exl3_linear_prefill(const uint16_t* xh, int rows, int n_sub, con
 // ---------------------------------------------------------------------------
 // exl3_linear_forward_static: the one-launch small-batch layer for callers that
 // cannot allocate device memory (code under HIP graph capture, serving loops,
-// harnesses that forbid hipMalloc). The split-K partial rows and the group
-// counters, which exl3_linear_forward takes from the caller, live in a
+// harnesses that forbid hipMalloc). The split-K accumulators, which
+// exl3_linear_forward takes from the caller (its counters argument), live in a
 // file-scope device array instead. Each GPU holds its own copy of the array at
 // its own address for the life of the process; the address is looked up once
 // per device and only that pointer is ever handed to a kernel (the array's name
 // is a host-side stand-in, not a device address).
 namespace exl3 {
 
-constexpr size_t kStaticCounterInts = 4096;              // 128-column groups: out <= 524288
-constexpr size_t kStaticPartialBytes = (size_t)16 << 20;  // fp32 split-K partial rows
-constexpr size_t kStaticScratchBytes = kStaticPartialBytes + kStaticCounterInts * sizeof(int32_t);
+constexpr size_t kStaticPartialBytes = (size_t)16 << 20;  // fp32 partial rows (large launches)
+constexpr size_t kStaticCounterBytes = (size_t)16 << 20;  // 64-bit accumulators / group counters
+constexpr size_t kStaticScratchBytes = kStaticPartialBytes + kStaticCounterBytes;
 constexpr int kStaticMaxDevices = 64;
 
 __global__ void static_zero_kernel(int32_t* p, int n) {
@@ -200,7 +201,8 @@ static __device__ __align__(256) unsigned char scratch[exl3::kStaticScratchBytes
 namespace exl3 {
 
 // Device address of this GPU's copy of `scratch` (resolved on first use, with that
-// device current); the counters in it are cleared once by a fill kernel on `stream`.
+// device current); the array is cleared once by a fill kernel on `stream` (every
+// launch leaves the accumulators it used at zero).
 static int static_scratch(hipStream_t stream, unsigned char** out) {
     static unsigned char* ptrs[kStaticMaxDevices];  // zero-initialised; one slot per device
     static std::mutex lock;
@@ -211,9 +213,9 @@ static int static_scratch(hipStream_t stream, unsigned char** out) {
     if (!ptrs[dev]) {
         void* p = nullptr;
         if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return EXL3_E_LAUNCH;
-        int32_t* counters = reinterpret_cast<int32_t*>(static_cast<unsigned char*>(p) + kStaticPartialBytes);
-        static_zero_kernel<<<dim3((unsigned)((kStaticCounterInts + 255) / 256)), dim3(256), 0, stream>>>(
-            counters, (int)kStaticCounterInts);
+        const int n_ints = (int)(kStaticCounterBytes / sizeof(int32_t));
+        static_zero_kernel<<<dim3((unsigned)((n_ints + 255) / 256)), dim3(256), 0, stream>>>(
+            reinterpret_cast<int32_t*>(static_cast<unsigned char*>(p) + kStaticPartialBytes), n_ints);
         if (int rc = launch_status()) return rc;
         ptrs[dev] = static_cast<unsigned char*>(p);
     }
@@ -229,6 +231,8 @@ EXL3_EXPORT size_t exl3_linear_static_need_bytes(int rows, int in_features, int 
     using namespace exl3;
     if (rows < 1 || rows > kLinearSmallMaxRows || in_features < 128 || out_features < 128) return 0;
     const GemvPlan plan = plan_linear_small(rows, in_features / 16, out_features / 128);
+    if (linear_small_uses_atomics(rows, out_features / 128, plan))
+        return linear_small_counter_ints(rows, out_features) * sizeof(int32_t);
     return (size_t)plan.n_partials() * rows * out_features * sizeof(float);
 }
 
@@ -245,10 +249,10 @@ EXL3_EXPORT int exl3_linear_forward_static(const uint16_t* x, int rows, const ui
     if (rows > kLinearSmallMaxRows) return EXL3_E_UNSUPPORTED;  // only the one-launch kernel
     if (n_sub > 1 && (!group_sub || !suh)) return EXL3_E_BAD_INDEX;
     const int n_groups = out_tiles / 8;
-    if ((size_t)n_groups > kStaticCounterInts) return EXL3_E_STATIC_LIMIT;
     const GemvPlan plan = plan_linear_small(rows, in_tiles, n_groups);
-    const size_t need = (size_t)plan.n_partials() * rows * out_tiles * 16 * sizeof(float);
-    if (need > kStaticPartialBytes) return EXL3_E_STATIC_LIMIT;
+    const size_t need = exl3_linear_static_need_bytes(rows, in_tiles * 16, out_tiles * 16);
+    if (need > kStaticPartialBytes || (size_t)n_groups * sizeof(int32_t) > kStaticCounterBytes)
+        return EXL3_E_STATIC_LIMIT;
     hipStream_t s = as_stream(stream);
     unsigned char* base = nullptr;
     if (int rc = static_scratch(s, &base)) return rc;

@@ -68,9 +68,18 @@ int launch_gemv_partials(const uint16_t* xh, int rows, int n_sub, const uint16_t
                          const int32_t* group_tile, int n_groups, float* partial, GemvPlan plan,
                          hipStream_t stream);
 
-// One-launch small-batch layer (rows <= kLinearSmallMaxRows): counters[out_tiles/8]
-// must be zero on entry and are zero again on exit. The kernel rotates x itself.
+// One-launch small-batch layer (rows <= kLinearSmallMaxRows). The kernel rotates x
+// itself. Its split reduction is one of two: 64-bit fixed-point accumulators
+// (uint64 [rows][16*out_tiles], living in `counters`, 8-byte aligned; `partial`
+// unused) when linear_small_uses_atomics(), else fp32 partial rows
+// [plan.n_partials()][rows][out] in `partial` plus counters[out_tiles/8]. Either way
+// the counters array must be zero on entry and is zero again on exit;
+// linear_small_counter_ints() is the length that serves both.
 constexpr int kLinearSmallMaxRows = kGemvMaxRows;
+bool linear_small_uses_atomics(int rows, int n_groups, GemvPlan plan);
+inline size_t linear_small_counter_ints(int rows, int out_features) {
+    return 2 * (size_t)rows * out_features;  // >= out_features / 128
+}
 int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, int in_tiles,
                         int out_tiles, int K, int cb, const uint16_t* suh, int n_sub,
                         const int32_t* group_sub, const uint16_t* svh, const uint16_t* bias,

@@ -176,17 +176,18 @@ __global__ __launch_bounds__(256) void gemv_kernel(
 //     current tile rows need, keeps the fp16 result in its own LDS slot and reads
 //     the 16 activations of a tile row back with two broadcast ds_read_b128; the
 //     raw block after that is already in flight while the current one is used;
-//   * output side: every wave stores its fp32 partial row, then bumps the
-//     counter of its 128-column group; the wave that brings the counter to
-//     n_splits adds the partials in split order, rounds to fp16 (the cast at
-//     ponyexl3/ref/forward.py:41), applies the output Hadamard of that one
-//     128-column block, svh and bias, and resets the counter to zero. No wave
-//     ever waits for another one, and the sum order is fixed, so the result is
-//     deterministic.
-// Counters must be zero on entry; they are zero again when the kernel ends.
+//   * output side: every workgroup adds its partial row to the accumulators of its
+//     128-column group with returning atomics (fixed point, so the total is
+//     independent of the arrival order); the workgroup whose add completes the group
+//     rounds to fp16 (the cast at ponyexl3/ref/forward.py:41), applies the output
+//     Hadamard of that one 128-column block, svh and bias, and zeroes the
+//     accumulators again. No workgroup waits for another one to be scheduled.
+// The counters array (accumulators uint64 [rows][out], or one int per column group)
+// must be zero on entry; it is zero again when the kernel ends.
 //
 // HALF (one and two rows only): splits are half blocks of four tile rows.
-template <int K, int CB, int MT, bool HALF>
+// ATOMIC: which of the two split reductions described at the end of the kernel runs.
+template <int K, int CB, int MT, bool HALF, bool ATOMIC>
 __global__ __launch_bounds__(256) void linear_small_kernel(
     const uint32_t* __restrict__ trellis, const half_t* __restrict__ x,
     const half_t* __restrict__ suh, const half_t* __restrict__ svh,
@@ -217,17 +218,29 @@ __global__ __launch_bounds__(256) void linear_small_kernel(
                                                  (size_t)in_features, rows, suh_row, xs[wave], lane,
                                                  acc);
 
-    // ---- the four waves of the workgroup are summed through LDS in wave order,
-    // the workgroup stores ONE fp32 partial row, and the last workgroup of the
-    // 128-column group finishes the columns.
-    // The eight XCDs have private L2 caches, so a device-scope release/acquire
-    // fence would write back / invalidate a whole L2 per workgroup. Instead the
-    // data that crosses workgroups (partials, counters) only ever moves through
-    // device-scope accesses, which bypass the non-coherent cache levels: the
-    // partial stores are waited for before the counter is bumped, and the
-    // finishing workgroup reads them back with device-scope loads.
+    // ---- the four waves of the workgroup are summed through LDS in wave order; the
+    // workgroup's partial row then goes into the column group's accumulators with
+    // returning 64-bit atomic adds, and the workgroup whose add completes the group
+    // applies the output transform.
+    //
+    // Accumulator word of one (batch row, column): count << 56 | sum, the sum a signed
+    // fixed-point number with 24 fraction bits. Integer addition is associative, so the
+    // total does not depend on the order in which workgroups arrive (run-to-run
+    // deterministic), and the returned old value tells a lane both how many partial
+    // rows are in and what they add up to: the usual chain of store, wait, counter,
+    // wait, reload (three memory round trips) becomes one round trip.
+    // The eight XCDs have private L2 caches; the atomics are device-scope operations
+    // that execute at the memory side, so no cache level has to be written back or
+    // invalidated.
+    // Finisher = the workgroup whose add brought (row 0, first column of the group) to
+    // wg_splits: exactly one. Usually its other adds were last as well and it holds all
+    // the totals. If another workgroup's adds were interleaved with its own, some of its
+    // returned values are short; every contributor has issued all its adds by then (its
+    // first one has landed), so the finisher re-reads the accumulators until all
+    // counts are complete - a wait for memory operations that are already in flight,
+    // not for another wave to be scheduled. Accumulators must be zero on entry; the
+    // finisher zeroes them again.
     __shared__ float red[4][MT][128];
-    __shared__ int last_flag;
     const int c0 = (lane >> 3) * 16 + (lane & 7);
 #pragma unroll
     for (int m = 0; m < MT; m++) {
@@ -235,85 +248,182 @@ __global__ __launch_bounds__(256) void linear_small_kernel(
         red[wave][m][c0 + 8] = acc[m][1];
     }
     __syncthreads();
-    const size_t out_total = (size_t)n_groups * 128;
-    const int wg_splits = (n_splits + 3) >> 2;  // partial rows per group
-    const size_t col = (size_t)g * 128 + 2 * lane;
-    if (wave == 0) {
+    if constexpr (ATOMIC) {
+        if (wave != 0) return;
+        unsigned long long* sums = reinterpret_cast<unsigned long long*>(counters);
+        const size_t out_total = (size_t)n_groups * 128;
+        const int wg_splits = (n_splits + 3) >> 2;  // partial rows per group
+        const size_t col = (size_t)g * 128 + 2 * lane;
+        constexpr float kFixScale = 16777216.f;         // 2^24
+        constexpr float kFixClamp = 262144.f;           // |partial| is clamped to 2^18 (fp16 ends at 65504)
+        auto to_word = [&](float v) -> unsigned long long {
+            v = fminf(fmaxf(v, -kFixClamp), kFixClamp);
+            const long long fixed = (long long)((double)v * (double)kFixScale);
+            return (1ull << 56) + (unsigned long long)fixed;
+        };
+        auto word_count = [](unsigned long long w) -> int {
+            return (int)((long long)(w + (1ull << 55)) >> 56);
+        };
+        auto word_value = [&](unsigned long long w) -> float {
+            const long long c = (long long)(w + (1ull << 55)) >> 56;
+            const long long fixed = (long long)(w - ((unsigned long long)c << 56));
+            return (float)((double)fixed * (1.0 / (double)kFixScale));
+        };
+        unsigned long long w0[MT], w1[MT];
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            w0[m] = w1[m] = 0;
+            if (m < rows) {
+                const float vx = ((red[0][m][2 * lane] + red[1][m][2 * lane]) + red[2][m][2 * lane]) +
+                                 red[3][m][2 * lane];
+                const float vy = ((red[0][m][2 * lane + 1] + red[1][m][2 * lane + 1]) +
+                                  red[2][m][2 * lane + 1]) + red[3][m][2 * lane + 1];
+                const unsigned long long ax = to_word(vx), ay = to_word(vy);
+                unsigned long long* slot = sums + (size_t)m * out_total + col;
+                w0[m] = __hip_atomic_fetch_add(slot, ax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + ax;
+                w1[m] = __hip_atomic_fetch_add(slot + 1, ay, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + ay;
+            }
+        }
+        // lane 0's first word is (row 0, first column of the group)
+        const int first_count = __builtin_amdgcn_readfirstlane(word_count(w0[0]));
+        if (first_count != wg_splits) return;
+        auto all_complete = [&]() {
+            bool ok = true;
+#pragma unroll
+            for (int m = 0; m < MT; m++)
+                if (m < rows) ok = ok && word_count(w0[m]) == wg_splits && word_count(w1[m]) == wg_splits;
+            return __ballot(ok) == ~0ull;
+        };
+        for (int spin = 0; !all_complete() && spin < (1 << 22); spin++) {
+#pragma unroll
+            for (int m = 0; m < MT; m++) {
+                if (m < rows) {
+                    const unsigned long long* slot = sums + (size_t)m * out_total + col;
+                    w0[m] = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    w1[m] = __hip_atomic_load(slot + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+        }
+        half2_t sv, bv;
+        if (svh) sv = *reinterpret_cast<const half2_t*>(svh + col);
+        if (bias) bv = *reinterpret_cast<const half2_t*>(bias + col);
 #pragma unroll
         for (int m = 0; m < MT; m++) {
             if (m < rows) {
-                float2_t v;
-                v.x = ((red[0][m][2 * lane] + red[1][m][2 * lane]) + red[2][m][2 * lane]) +
-                      red[3][m][2 * lane];
-                v.y = ((red[0][m][2 * lane + 1] + red[1][m][2 * lane + 1]) +
-                       red[2][m][2 * lane + 1]) + red[3][m][2 * lane + 1];
-                uint64_t* dst = reinterpret_cast<uint64_t*>(
-                    partial + ((size_t)blockIdx.y * rows + m) * out_total + col);
-                __hip_atomic_store(dst, __builtin_bit_cast(uint64_t, v), __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
+                unsigned long long* slot = sums + (size_t)m * out_total + col;
+                __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(slot + 1, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                // the cast at ponyexl3/ref/forward.py:41, then the output Hadamard of this one
+                // 128-column block, svh and bias (forward.py:42-45)
+                float a = (float)(half_t)word_value(w0[m]);
+                float b = (float)(half_t)word_value(w1[m]);
+                wht128_lanes(a, b, lane);
+                a = __fmul_rn(a, kHadScaleF);
+                b = __fmul_rn(b, kHadScaleF);
+                if (svh) {
+                    a = __fmul_rn(a, (float)sv.x);
+                    b = __fmul_rn(b, (float)sv.y);
+                }
+                half2_t o;
+                o.x = (half_t)a;
+                o.y = (half_t)b;
+                if (bias) {
+                    o.x = o.x + bv.x;
+                    o.y = o.y + bv.y;
+                }
+                *reinterpret_cast<half2_t*>(y + (size_t)m * out_total + col) = o;
             }
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        int seen = 0;
-        if (lane == 0) {
-            seen = __hip_atomic_fetch_add(&counters[g], 1, __ATOMIC_RELAXED,
-                                          __HIP_MEMORY_SCOPE_AGENT);
-            last_flag = seen == wg_splits - 1;
+    } else {
+        // Few, large launches (many column groups x partial rows x batch rows): the
+        // memory side retires about 75 000 such atomics per microsecond, which costs
+        // more than the round trips it saves. There the partial row is stored, the
+        // group counter bumped, and the workgroup that brings it to wg_splits reloads
+        // the partial rows in index order. Partial rows and counters only ever move
+        // through device-scope accesses (the XCDs have private L2s; a release/acquire
+        // fence per workgroup would write back / invalidate a whole L2), and the
+        // stores are waited for (s_waitcnt vmcnt(0)) before the counter is bumped.
+        __shared__ int last_flag;
+        const size_t out_total = (size_t)n_groups * 128;
+        const int wg_splits = (n_splits + 3) >> 2;  // partial rows per group
+        const size_t col = (size_t)g * 128 + 2 * lane;
+        if (wave == 0) {
+#pragma unroll
+            for (int m = 0; m < MT; m++) {
+                if (m < rows) {
+                    float2_t v;
+                    v.x = ((red[0][m][2 * lane] + red[1][m][2 * lane]) + red[2][m][2 * lane]) +
+                          red[3][m][2 * lane];
+                    v.y = ((red[0][m][2 * lane + 1] + red[1][m][2 * lane + 1]) +
+                           red[2][m][2 * lane + 1]) + red[3][m][2 * lane + 1];
+                    uint64_t* dst = reinterpret_cast<uint64_t*>(
+                        partial + ((size_t)blockIdx.y * rows + m) * out_total + col);
+                    __hip_atomic_store(dst, __builtin_bit_cast(uint64_t, v), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            int seen = 0;
+            if (lane == 0) {
+                seen = __hip_atomic_fetch_add(&counters[g], 1, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
+                last_flag = seen == wg_splits - 1;
+            }
         }
-    }
-    __syncthreads();
-    if (!last_flag) return;
-    asm volatile("" ::: "memory");
-    half2_t sv, bv;
-    if (svh) sv = *reinterpret_cast<const half2_t*>(svh + col);
-    if (bias) bv = *reinterpret_cast<const half2_t*>(bias + col);
-    for (int m = wave; m < rows; m += 4) {  // the finishing workgroup splits the batch rows
-        // device-scope loads, sixteen partial rows in flight, added in split order
-        const float* src = partial + (size_t)m * out_total + col;
-        const size_t stride = (size_t)rows * out_total;
-        float a = 0.f, b = 0.f;
-        int s = 0;
-        for (; s + 16 <= wg_splits; s += 16) {
-            uint64_t v[16];
+        __syncthreads();
+        if (!last_flag) return;
+        asm volatile("" ::: "memory");
+        half2_t sv, bv;
+        if (svh) sv = *reinterpret_cast<const half2_t*>(svh + col);
+        if (bias) bv = *reinterpret_cast<const half2_t*>(bias + col);
+        for (int m = wave; m < rows; m += 4) {  // the finishing workgroup splits the batch rows
+            // device-scope loads, sixteen partial rows in flight, added in split order
+            const float* src = partial + (size_t)m * out_total + col;
+            const size_t stride = (size_t)rows * out_total;
+            float a = 0.f, b = 0.f;
+            int s = 0;
+            for (; s + 16 <= wg_splits; s += 16) {
+                uint64_t v[16];
 #pragma unroll
-            for (int i = 0; i < 16; i++)
-                v[i] = __hip_atomic_load(
-                    reinterpret_cast<const uint64_t*>(src + (size_t)(s + i) * stride),
-                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (int i = 0; i < 16; i++)
+                    v[i] = __hip_atomic_load(
+                        reinterpret_cast<const uint64_t*>(src + (size_t)(s + i) * stride),
+                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const float2_t f = __builtin_bit_cast(float2_t, v[i]);
+                for (int i = 0; i < 16; i++) {
+                    const float2_t f = __builtin_bit_cast(float2_t, v[i]);
+                    a = __fadd_rn(a, f.x);
+                    b = __fadd_rn(b, f.y);
+                }
+            }
+            for (; s < wg_splits; s++) {
+                const float2_t f = __builtin_bit_cast(
+                    float2_t, __hip_atomic_load(reinterpret_cast<const uint64_t*>(src + (size_t)s * stride),
+                                                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
                 a = __fadd_rn(a, f.x);
                 b = __fadd_rn(b, f.y);
             }
+            a = (float)(half_t)a;
+            b = (float)(half_t)b;
+            wht128_lanes(a, b, lane);
+            a = __fmul_rn(a, kHadScaleF);
+            b = __fmul_rn(b, kHadScaleF);
+            if (svh) {
+                a = __fmul_rn(a, (float)sv.x);
+                b = __fmul_rn(b, (float)sv.y);
+            }
+            half2_t o;
+            o.x = (half_t)a;
+            o.y = (half_t)b;
+            if (bias) {
+                o.x = o.x + bv.x;
+                o.y = o.y + bv.y;
+            }
+            *reinterpret_cast<half2_t*>(y + (size_t)m * out_total + col) = o;
         }
-        for (; s < wg_splits; s++) {
-            const float2_t f = __builtin_bit_cast(
-                float2_t, __hip_atomic_load(reinterpret_cast<const uint64_t*>(src + (size_t)s * stride),
-                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-            a = __fadd_rn(a, f.x);
-            b = __fadd_rn(b, f.y);
-        }
-        a = (float)(half_t)a;
-        b = (float)(half_t)b;
-        wht128_lanes(a, b, lane);
-        a = __fmul_rn(a, kHadScaleF);
-        b = __fmul_rn(b, kHadScaleF);
-        if (svh) {
-            a = __fmul_rn(a, (float)sv.x);
-            b = __fmul_rn(b, (float)sv.y);
-        }
-        half2_t o;
-        o.x = (half_t)a;
-        o.y = (half_t)b;
-        if (bias) {
-            o.x = o.x + bv.x;
-            o.y = o.y + bv.y;
-        }
-        *reinterpret_cast<half2_t*>(y + (size_t)m * out_total + col) = o;
+        if (threadIdx.x == 0)
+            __hip_atomic_store(&counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (threadIdx.x == 0)
-        __hip_atomic_store(&counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // y[i] = sum over the partial rows, index order.
@@ -369,6 +479,17 @@ GemvPlan plan_linear_small(int rows, int in_tiles, int n_groups) {
     return GemvPlan{n_splits, blocks_per_split * 8};
 }
 
+// The atomic-accumulator reduction pays off while the launch issues few atomics:
+// (column groups x partial rows per group x 128 columns x batch rows). Measured on
+// the 27B-class shapes at one row: 33 k (4096 -> 4096) 9.1 -> 6.8 us, q+k+v
+// 15.0 -> 13.2 us (205 k with half-block splits), 174 k (down) 20.7 -> 19.2 us, 348 k (gate+up) no gain; at 8 rows
+// (2.8 M) the step got 13 % slower.
+bool linear_small_uses_atomics(int rows, int n_groups, GemvPlan plan) {
+    static const int kMaxAtomics = env_int("EXL3_LINEAR_MAX_ATOMICS", 300000, 0, 1 << 30);
+    if (plan.n_partials() > 255) return false;  // the count field has eight bits
+    return (long long)n_groups * plan.n_partials() * 128 * rows <= kMaxAtomics;
+}
+
 int launch_gemv_partials(const uint16_t* xh, int rows, int n_sub, const uint16_t* trellis,
                          int in_tiles, int out_tiles, int K, int cb, const int32_t* group_sub,
                          const int32_t* group_tile, int n_groups, float* partial, GemvPlan plan,
@@ -408,7 +529,10 @@ int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, in
                         uint16_t* y, float* partial, int* counters, GemvPlan plan,
                         hipStream_t stream) {
     if (int rc = check_k_cb(K, cb)) return rc;
-    if (!x || !trellis || !y || !partial || !counters) return EXL3_E_NULL_POINTER;
+    if (!x || !trellis || !y || !counters) return EXL3_E_NULL_POINTER;
+    const bool atomic = linear_small_uses_atomics(rows, out_tiles / 8, plan);
+    if (atomic && (reinterpret_cast<uintptr_t>(counters) & 7)) return EXL3_E_BAD_SHAPE;
+    if (!atomic && !partial) return EXL3_E_NULL_POINTER;
     if (rows < 1 || rows > kLinearSmallMaxRows || n_sub < 1 || in_tiles < 8 || out_tiles < 8 ||
         in_tiles % 8 || out_tiles % 8)
         return EXL3_E_BAD_SHAPE;
@@ -423,13 +547,17 @@ int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, in
     const int mt = rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8;
     return dispatch_k_cb(K, cb, [&](auto k, auto c) {
         auto go = [&](auto mtc, auto halfc) {
-            linear_small_kernel<k.value, c.value, mtc.value, halfc.value>
-                <<<grid, dim3(256), 0, stream>>>(
-                    reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<const half_t*>(x),
-                    reinterpret_cast<const half_t*>(suh), reinterpret_cast<const half_t*>(svh),
-                    reinterpret_cast<const half_t*>(bias), reinterpret_cast<half_t*>(y), partial,
-                    counters, group_sub, in_tiles, out_tiles, rows, n_groups, plan.tk_per_split,
-                    plan.n_splits);
+            auto launch = [&](auto atomicc) {
+                linear_small_kernel<k.value, c.value, mtc.value, halfc.value, atomicc.value>
+                    <<<grid, dim3(256), 0, stream>>>(
+                        reinterpret_cast<const uint32_t*>(trellis),
+                        reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(suh),
+                        reinterpret_cast<const half_t*>(svh), reinterpret_cast<const half_t*>(bias),
+                        reinterpret_cast<half_t*>(y), partial, counters, group_sub, in_tiles,
+                        out_tiles, rows, n_groups, plan.tk_per_split, plan.n_splits);
+            };
+            if (atomic) launch(std::true_type{});
+            else launch(std::false_type{});
         };
         using T = std::true_type;
         using F = std::false_type;

@@ -627,7 +627,10 @@ def linear_forward(x2d, trellis, k, cb, suh=None, svh=None, bias=None, group_sub
     lib = _lib.load()
     ws_bytes = int(lib.exl3_linear_workspace_bytes(rows, n_in, n_out, n_sub))
     ws = workspace(x2d.device, ws_bytes)
-    cnt = sync_counters(x2d.device, n_out // 128) if fused else None
+    # one-launch kernel: a 64-bit accumulator per (row, output column) = two ints each;
+    # medium-batch kernel: one counter per 128-column group
+    n_cnt = 2 * rows * n_out if rows <= gemv_max_rows() else n_out // 128
+    cnt = sync_counters(x2d.device, n_cnt) if fused else None
     rc = lib.exl3_linear_forward(
         _ptr(x2d), rows, _ptr(trellis), in_tiles, out_tiles, int(k), int(cb), _ptr(suh), n_sub,
         _ptr(group_sub), _ptr(svh), _ptr(bias), _ptr(y), _ptr(ws), ws.numel(), _ptr(cnt),

@@ -40,7 +40,7 @@ def _forward_pair(lib, cuda, x, t, k, cb, suh, svh, bias):
     n_out = out_tiles * 16
     ws_bytes = int(lib.exl3_linear_workspace_bytes(rows, n_in, n_out, 1))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
-    cnt = torch.zeros(n_out // 128, dtype=torch.int32, device=cuda)
+    cnt = torch.zeros(2 * rows * n_out, dtype=torch.int32, device=cuda)  # 64-bit accumulators
     y_ref = torch.empty((rows, n_out), dtype=torch.float16, device=cuda)
     rc = lib.exl3_linear_forward(_ptr(x), rows, _ptr(t), in_tiles, out_tiles, k, cb, _ptr(suh), 1, None,
                                  _ptr(svh), _ptr(bias), _ptr(y_ref), _ptr(ws), ws.numel(), _ptr(cnt),
@@ -62,7 +62,7 @@ def test_static_entry_matches_workspace_entry_twice(cuda, oracle):
     lib = L.load()
     assert int(lib.exl3_linear_static_scratch_bytes()) == 16 << 20
     rng = np.random.default_rng(5)
-    # first call: many split partial rows (2176 x 640, 4 rows); second: a smaller layer, 1 row
+    # first call: many workgroups per column group (2176 x 640, 4 rows); second: a smaller layer, 1 row
     for (k, mcg, n_in, n_out, rows, seed) in [(4, False, 2176, 640, 4, 3), (3, True, 256, 384, 1, 4)]:
         print(f"static entry k={k} mcg={mcg} {n_in}x{n_out} rows={rows}", flush=True)
         layer, t, suh, svh, b = _layer_tensors(cuda, k, n_in, n_out, seed, mcg=mcg, bias=True)
@@ -88,8 +88,8 @@ def test_static_entry_rejects_what_does_not_fit(cuda):
     rc = lib.exl3_linear_forward_static(_ptr(x), 9, _ptr(t), 16, 16, 4, 0, None, 1, None, None, None,
                                         _ptr(y), _stream())
     assert rc == L.EXL3_E_UNSUPPORTED
-    # a shape whose partial rows exceed the built-in scratch: only sizes are looked at,
-    # so the (too small) buffers are never touched
+    # a shape whose accumulators (8 bytes per row and output column) exceed the built-in
+    # scratch: only sizes are looked at, so the (too small) buffers are never touched
     in_tiles, out_tiles = 4096, 65536
     assert int(lib.exl3_linear_static_need_bytes(8, in_tiles * 16, out_tiles * 16)) > 16 << 20
     rc = lib.exl3_linear_forward_static(_ptr(x), 8, _ptr(t), in_tiles, out_tiles, 4, 0, None, 1, None,
