@@ -56,8 +56,9 @@ constexpr int kGemvMaxRows = 8;
 struct GemvPlan {
     int n_splits;      // wave-level splits of the tile rows
     int tk_per_split;  // tile rows per split
-    // the four waves of a workgroup are summed in LDS: partial rows per group
-    int n_partials() const { return (n_splits + 3) / 4; }
+    int wg_waves = 4;  // waves per workgroup (4; the one-launch layer kernel also has 8)
+    // the waves of a workgroup are summed in LDS: partial rows per group
+    int n_partials() const { return (n_splits + wg_waves - 1) / wg_waves; }
 };
 GemvPlan plan_gemv(int rows, int in_tiles, int n_groups);
 GemvPlan plan_linear_small(int rows, int in_tiles, int n_groups);
@@ -77,6 +78,9 @@ int launch_gemv_partials(const uint16_t* xh, int rows, int n_sub, const uint16_t
 // linear_small_counter_ints() is the length that serves both.
 constexpr int kLinearSmallMaxRows = kGemvMaxRows;
 bool linear_small_uses_atomics(int rows, int n_groups, GemvPlan plan);
+// plan_linear_small with the reduction in mind: one row on a large layer takes
+// workgroups of eight waves when that brings the launch under the atomics limit.
+GemvPlan plan_linear_small_launch(int rows, int in_tiles, int n_groups);
 inline size_t linear_small_counter_ints(int rows, int out_features) {
     return 2 * (size_t)rows * out_features;  // >= out_features / 128
 }

@@ -187,18 +187,21 @@ __global__ __launch_bounds__(256) void gemv_kernel(
 //
 // HALF (one and two rows only): splits are half blocks of four tile rows.
 // ATOMIC: which of the two split reductions described at the end of the kernel runs.
-template <int K, int CB, int MT, bool HALF, bool ATOMIC>
-__global__ __launch_bounds__(256) void linear_small_kernel(
+// NW: waves per workgroup, 4 or 8 (8 only with ATOMIC: half as many workgroups add
+// to a column group's accumulators).
+template <int K, int CB, int MT, bool HALF, bool ATOMIC, int NW = 4>
+__global__ __launch_bounds__(NW * 64) void linear_small_kernel(
     const uint32_t* __restrict__ trellis, const half_t* __restrict__ x,
     const half_t* __restrict__ suh, const half_t* __restrict__ svh,
     const half_t* __restrict__ bias, half_t* __restrict__ y, float* partial, int* counters,
     const int* __restrict__ group_sub, int in_tiles, int out_tiles, int rows, int n_groups,
     int tk_per_split, int n_splits) {
-    __shared__ __attribute__((aligned(16))) half_t xs[4][MT][kXwLd];
+    static_assert(NW == 4 || (NW == 8 && ATOMIC), "eight-wave workgroups use the accumulators");
+    __shared__ __attribute__((aligned(16))) half_t xs[NW][MT][kXwLd];
     const int g = blockIdx.x;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int split = blockIdx.y * 4 + wave;
+    const int split = blockIdx.y * NW + wave;
     const bool active = split < n_splits;  // idle waves still take part in the barriers below
     const int sub = group_sub ? group_sub[g] : 0;
     const int in_features = in_tiles * 16;
@@ -240,7 +243,7 @@ __global__ __launch_bounds__(256) void linear_small_kernel(
     // counts are complete - a wait for memory operations that are already in flight,
     // not for another wave to be scheduled. Accumulators must be zero on entry; the
     // finisher zeroes them again.
-    __shared__ float red[4][MT][128];
+    __shared__ float red[NW][MT][128];
     const int c0 = (lane >> 3) * 16 + (lane & 7);
 #pragma unroll
     for (int m = 0; m < MT; m++) {
@@ -252,7 +255,7 @@ __global__ __launch_bounds__(256) void linear_small_kernel(
         if (wave != 0) return;
         unsigned long long* sums = reinterpret_cast<unsigned long long*>(counters);
         const size_t out_total = (size_t)n_groups * 128;
-        const int wg_splits = (n_splits + 3) >> 2;  // partial rows per group
+        const int wg_splits = (n_splits + NW - 1) / NW;  // partial rows per group
         const size_t col = (size_t)g * 128 + 2 * lane;
         constexpr float kFixScale = 16777216.f;         // 2^24
         constexpr float kFixClamp = 262144.f;           // |partial| is clamped to 2^18 (fp16 ends at 65504)
@@ -274,10 +277,12 @@ __global__ __launch_bounds__(256) void linear_small_kernel(
         for (int m = 0; m < MT; m++) {
             w0[m] = w1[m] = 0;
             if (m < rows) {
-                const float vx = ((red[0][m][2 * lane] + red[1][m][2 * lane]) + red[2][m][2 * lane]) +
-                                 red[3][m][2 * lane];
-                const float vy = ((red[0][m][2 * lane + 1] + red[1][m][2 * lane + 1]) +
-                                  red[2][m][2 * lane + 1]) + red[3][m][2 * lane + 1];
+                float vx = red[0][m][2 * lane], vy = red[0][m][2 * lane + 1];
+#pragma unroll
+                for (int w = 1; w < NW; w++) {  // wave order
+                    vx = __fadd_rn(vx, red[w][m][2 * lane]);
+                    vy = __fadd_rn(vy, red[w][m][2 * lane + 1]);
+                }
                 const unsigned long long ax = to_word(vx), ay = to_word(vy);
                 unsigned long long* slot = sums + (size_t)m * out_total + col;
                 w0[m] = __hip_atomic_fetch_add(slot, ax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + ax;
@@ -490,6 +495,16 @@ bool linear_small_uses_atomics(int rows, int n_groups, GemvPlan plan) {
     return (long long)n_groups * plan.n_partials() * 128 * rows <= kMaxAtomics;
 }
 
+GemvPlan plan_linear_small_launch(int rows, int in_tiles, int n_groups) {
+    GemvPlan plan = plan_linear_small(rows, in_tiles, n_groups);
+    if (rows == 1 && plan.tk_per_split >= 8 && !linear_small_uses_atomics(rows, n_groups, plan)) {
+        GemvPlan wide = plan;
+        wide.wg_waves = 8;
+        if (linear_small_uses_atomics(rows, n_groups, wide)) plan = wide;
+    }
+    return plan;
+}
+
 int launch_gemv_partials(const uint16_t* xh, int rows, int n_sub, const uint16_t* trellis,
                          int in_tiles, int out_tiles, int K, int cb, const int32_t* group_sub,
                          const int32_t* group_tile, int n_groups, float* partial, GemvPlan plan,
@@ -543,7 +558,9 @@ int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, in
         (long long)plan.n_splits * plan.tk_per_split < in_tiles)
         return EXL3_E_BAD_SHAPE;
     const int n_groups = out_tiles / 8;
-    const dim3 grid((unsigned)n_groups, (unsigned)((plan.n_splits + 3) / 4));
+    if (plan.wg_waves != 4 && !(plan.wg_waves == 8 && rows == 1 && !half && atomic))
+        return EXL3_E_UNSUPPORTED;
+    const dim3 grid((unsigned)n_groups, (unsigned)plan.n_partials());
     const int mt = rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8;
     return dispatch_k_cb(K, cb, [&](auto k, auto c) {
         auto go = [&](auto mtc, auto halfc) {
@@ -559,6 +576,16 @@ int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, in
             if (atomic) launch(std::true_type{});
             else launch(std::false_type{});
         };
+        if (plan.wg_waves == 8) {  // one row, whole blocks, accumulators (checked above)
+            linear_small_kernel<k.value, c.value, 1, false, true, 8>
+                <<<grid, dim3(512), 0, stream>>>(
+                    reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<const half_t*>(x),
+                    reinterpret_cast<const half_t*>(suh), reinterpret_cast<const half_t*>(svh),
+                    reinterpret_cast<const half_t*>(bias), reinterpret_cast<half_t*>(y), partial,
+                    counters, group_sub, in_tiles, out_tiles, rows, n_groups, plan.tk_per_split,
+                    plan.n_splits);
+            return launch_status();
+        }
         using T = std::true_type;
         using F = std::false_type;
         switch (mt) {
