@@ -593,7 +593,9 @@ def bench_encoder(dev):
 
 
 def bench_moe(dev):
-    """config 4: A3B-style routed experts, top-8 of 256, 1 and 8 tokens."""
+    """config 4: A3B-style routed experts, top-8 of 256, at 1, 8 and 32 tokens (from
+    16 tokens on the slots of one expert share a pass over its weights) and 512
+    tokens through the prefill path."""
     import torch
 
     from ponyexl3_amd import EXL3SwitchGLU, ops
@@ -613,7 +615,7 @@ def bench_moe(dev):
             k=K_BITS, cb=CB))
     res = {}
     per_graph = 32  # chains per graph, each with its own routing, alternating weight copies
-    for T in (1, 8):
+    for T in (1, 8, 32):
         x = torch.from_numpy((rng.standard_normal((1, T, D)) * 0.25).astype(np.float16)).to(dev)
         # Routing differs from chain to chain so that a replay streams far more expert
         # weights than the 256 MB last-level cache holds: at one token the 32 chains

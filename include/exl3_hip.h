@@ -302,7 +302,8 @@ int exl3_linear_forward_static(const uint16_t *x, int rows, const uint16_t *trel
                                uint16_t *y, void *stream);
 
 /*
- * Routed MoE expert chain for rows <= 8 tokens (EXL3SwitchGLU.__call__,
+ * Routed MoE expert chain for a handful of tokens, tokens*top_k <= 4096 slots
+ * (EXL3SwitchGLU.__call__ at rows <= 8 in the reference,
  * ponyexl3/mlx/exl3_moe.py:770-787; unfused definition :648-682):
  * per slot (token t, expert e = indices[t][s]):
  *   g = L_gate,e(x_t); u = L_up,e(x_t); h = fp16(act(g) * u); y = L_down,e(h)
@@ -321,7 +322,10 @@ int exl3_linear_forward_static(const uint16_t *x, int rows, const uint16_t *trel
  *               A2/B2 pair (ponyexl3/mlx/exl3_moe.py:345-422: gate/up, then
  *               GLU + rotation + down); without, five launches that need no
  *               state between calls. Calls that overlap on one counters array race.
- * Only the selected experts' trellis blocks are read.
+ * Only the selected experts' trellis blocks are read. In the two-launch chain, with
+ * 2 <= tokens, at most 512 slots and at least one slot per two experts, the slots that
+ * route to one expert share a pass over its weights (four batch rows per pass; same
+ * arithmetic per row, bit-identical results); EXL3_MOE_GROUP=0 switches that off.
  */
 int exl3_moe_forward(const uint16_t *x, int tokens, const int32_t *indices, int top_k,
                      const uint16_t *gu_trellis, const uint16_t *gu_suh, const uint16_t *gu_svh,

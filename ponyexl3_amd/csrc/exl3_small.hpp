@@ -22,6 +22,16 @@ __device__ __forceinline__ void load_lane_words_nt(const uint32_t* __restrict__ 
     for (int i = 0; i < K; i++) own[i] = __builtin_nontemporal_load(p + i);
 }
 
+// The same through a pointer that is declared to be in global memory (for addresses
+// whose origin the compiler cannot see; it would otherwise emit flat loads).
+using global_words_t = const uint32_t __attribute__((address_space(1)))*;
+
+template <int K>
+__device__ __forceinline__ void load_lane_words_nt(global_words_t p, uint32_t (&own)[K]) {
+#pragma unroll
+    for (int i = 0; i < K; i++) own[i] = __builtin_nontemporal_load(p + i);
+}
+
 // Unnormalised WHT over 128 values held as (a, b) = elements (2*lane, 2*lane+1);
 // same butterfly order as ponyexl3/ref/hadamard.py:16-30 (stage h pairs i, i+h).
 __device__ __forceinline__ void wht128_lanes(float& a, float& b, int lane) {
@@ -54,26 +64,46 @@ __device__ __forceinline__ void wht128_lanes(float& a, float& b, int lane) {
 // HALF: the range is one half of a block, [tk_begin, tk_begin + 4) with tk_begin a
 // multiple of 4. The wave still rotates (or stages) the whole 128-wide block, then
 // uses four of its eight tile rows. Narrow layers get twice the waves this way.
-template <int K, int CB, int MT, bool ROTATE, bool HALF = false>
-__device__ __forceinline__ void stream_block_rows(const uint32_t* __restrict__ base,
-                                                  size_t row_words, int tk_begin, int tk_end,
-                                                  const half_t* __restrict__ x, size_t x_stride,
-                                                  int rows, const half_t* __restrict__ suh_row,
-                                                  half_t (*xw)[kXwLd], int lane,
-                                                  float (&acc)[MT][2]) {
+//
+// The batch rows are given by address (xrow[m], m < MT; entries past `rows` repeat a
+// valid row), so that a caller can gather them. GUARD: rows past `rows` are neither
+// loaded nor rotated (their LDS rows and sums are then meaningless and must not be
+// used). PRELOADED: the caller has already issued the first trellis loads into `buf`
+// with issue_first_rows (to overlap their latency with work of its own).
+constexpr int kStreamSlots = 4;  // wave-wide loads in flight (divides the 8 steps of a block)
+
+template <int K, bool HALF, class Words>
+__device__ __forceinline__ void issue_first_rows(Words base, size_t row_words, int tk_begin,
+                                                 int tk_end, uint32_t (&buf)[kStreamSlots][K]) {
+#pragma unroll
+    for (int s = 0; s < kStreamSlots; s++) {
+        const int tk = HALF ? tk_begin + s : min(tk_begin + s, tk_end - 1);
+        load_lane_words_nt<K>(base + (size_t)tk * row_words, buf[s]);
+    }
+}
+
+template <int K, int CB, int MT, bool ROTATE, bool HALF, bool GUARD, bool PRELOADED>
+__device__ __forceinline__ void stream_block_rows_at(const uint32_t* __restrict__ base,
+                                                     size_t row_words, int tk_begin, int tk_end,
+                                                     const half_t* const (&xrow)[MT], int rows,
+                                                     const half_t* __restrict__ suh_row,
+                                                     half_t (*xw)[kXwLd], int lane,
+                                                     float (&acc)[MT][2],
+                                                     uint32_t (&buf)[kStreamSlots][K]) {
     half2_t xraw[MT], sraw;
     auto fetch_block = [&](int blk) {
         const int off = blk * 128 + 2 * lane;
 #pragma unroll
         for (int m = 0; m < MT; m++) {
-            const int r = m < rows ? m : 0;
-            xraw[m] = *reinterpret_cast<const half2_t*>(x + (size_t)r * x_stride + off);
+            if (GUARD && m >= rows) break;
+            xraw[m] = *reinterpret_cast<const half2_t*>(xrow[m] + off);
         }
         if (ROTATE && suh_row) sraw = *reinterpret_cast<const half2_t*>(suh_row + off);
     };
     auto stage_block = [&]() {
 #pragma unroll
         for (int m = 0; m < MT; m++) {
+            if (GUARD && m >= rows) break;
             half2_t o = xraw[m];
             if constexpr (ROTATE) {
                 float a = (float)xraw[m].x, b = (float)xraw[m].y;
@@ -142,13 +172,10 @@ __device__ __forceinline__ void stream_block_rows(const uint32_t* __restrict__ b
             }
         }
     };
-    constexpr int kSlots = 4;  // wave-wide loads in flight (divides the 8 steps of a block)
-    uint32_t buf[kSlots][K];
+    constexpr int kSlots = kStreamSlots;
+    if constexpr (!PRELOADED) issue_first_rows<K, HALF>(base, row_words, tk_begin, tk_end, buf);
     if constexpr (HALF) {
         // all four loads up front, no refills
-#pragma unroll
-        for (int s = 0; s < kSlots; s++)
-            load_lane_words_nt<K>(base + (size_t)(tk_begin + s) * row_words, buf[s]);
         fetch_block(tk_begin >> 3);
         stage_block();
         const int row0 = tk_begin & 7;  // 0 or 4
@@ -172,9 +199,6 @@ __device__ __forceinline__ void stream_block_rows(const uint32_t* __restrict__ b
     }
     // Ranges are whole blocks, so the staging sits outside the unrolled 8-step
     // pipeline and the LDS offsets of the activations are compile-time constants.
-#pragma unroll
-    for (int s = 0; s < kSlots; s++)
-        load_lane_words_nt<K>(base + (size_t)min(tk_begin + s, tk_end - 1) * row_words, buf[s]);
     fetch_block(tk_begin >> 3);
     uint32_t prev = neighbour_word(buf[0][K - 1], lane);
     for (int tkb = tk_begin; tkb < tk_end; tkb += 8) {
@@ -199,6 +223,22 @@ __device__ __forceinline__ void stream_block_rows(const uint32_t* __restrict__ b
         acc[m][0] += accv[0][m >> 2][m & 3];
         acc[m][1] += accv[1][m >> 2][m & 3];
     }
+}
+
+// The same over `rows` consecutive rows of a row-major activation matrix.
+template <int K, int CB, int MT, bool ROTATE, bool HALF = false>
+__device__ __forceinline__ void stream_block_rows(const uint32_t* __restrict__ base,
+                                                  size_t row_words, int tk_begin, int tk_end,
+                                                  const half_t* __restrict__ x, size_t x_stride,
+                                                  int rows, const half_t* __restrict__ suh_row,
+                                                  half_t (*xw)[kXwLd], int lane,
+                                                  float (&acc)[MT][2]) {
+    const half_t* xrow[MT];
+#pragma unroll
+    for (int m = 0; m < MT; m++) xrow[m] = x + (size_t)(m < rows ? m : 0) * x_stride;
+    uint32_t buf[kStreamSlots][K];
+    stream_block_rows_at<K, CB, MT, ROTATE, HALF, false, false>(
+        base, row_words, tk_begin, tk_end, xrow, rows, suh_row, xw, lane, acc, buf);
 }
 
 }  // namespace exl3

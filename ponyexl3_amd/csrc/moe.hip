@@ -16,6 +16,8 @@
 //                           the rotated block, sum, post-Hadamard, svh
 //   (four waves per workgroup, one Hadamard block of the reduction each; with few
 //   slots eight waves on half a block each, which doubles the loads in flight)
+//   With several tokens and enough slots per expert (moe_*_grouped_kernel) the slots
+//   that route to one expert share a pass over its weights, four batch rows at a time.
 // Without counters the same result comes from a chain of five launches:
 //   1. moe_prep_kernel      rotated activations per (slot, proj) + group tables
 //   2. gemv_kernel          gate/up partial sums, fp32
@@ -347,6 +349,288 @@ __global__ __launch_bounds__(NW * 64) void moe_down_kernel(
     *reinterpret_cast<half2_t*>(y + (size_t)s * D + og * 128 + 2 * lane) = o;
 }
 
+// ---------------------------------------------------------------------------
+// The same chain with the slots grouped by expert. With several tokens, slots that
+// route to the same expert share one pass over its weights: the grid stays one
+// workgroup set per slot, every workgroup finds the slots of its own expert in the
+// routing table, and only the first of every four of them (in slot order) works, on up
+// to four batch rows (the 4x4x4 matrix instructions carry four rows at the price of
+// one). The others leave at once. Per row the arithmetic, the partial rows and the
+// counters are those of the kernels above, so the results are bit-identical.
+
+constexpr int kGroupRows = 4;       // batch rows one workgroup carries
+constexpr int kGroupMaxSlots = 512; // routing table entries a workgroup scans (8 per lane)
+
+struct SlotGroup {
+    int n;               // rows of this workgroup; 0 = another workgroup carries this slot
+    int expert;
+    int s0, s1, s2, s3;  // the rows' slots, ascending; entries past n repeat s0
+};
+
+// Loads above stay above, work below stays below (in the optimiser, which would sink
+// loads to their first use, and in the instruction scheduler): the routing table is
+// requested first, the first trellis rows second, and the search of the table runs
+// while the trellis rows are in flight. Emits no instruction.
+__device__ __forceinline__ void pin_program_order() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// The same address with its origin hidden from the optimiser: loads through a kernel
+// argument that is declared free of aliases may otherwise move across pin_program_order.
+__device__ __forceinline__ global_words_t opaque_pointer(const uint32_t* p) {
+    asm volatile("" : "+v"(p));
+    return (global_words_t)p;
+}
+
+// A wave's copy of the routing table: lane l holds entries c*64 + l (the last entry
+// repeated past the end). Always the same number of loads, whatever `slots` is, so
+// that the wait for them can leave younger loads in flight.
+struct SlotTable {
+    int idx[kGroupMaxSlots / 64];
+};
+
+__device__ __forceinline__ SlotTable load_slot_table(const int* __restrict__ indices, int slots,
+                                                     int lane) {
+    SlotTable t;
+#pragma unroll
+    for (int c = 0; c < kGroupMaxSlots / 64; c++) t.idx[c] = indices[min(c * 64 + lane, slots - 1)];
+    return t;
+}
+
+// Nothing computed from the table may be placed above this point.
+__device__ __forceinline__ void use_table_from_here(SlotTable& t) {
+#pragma unroll
+    for (int c = 0; c < kGroupMaxSlots / 64; c++) asm volatile("" : "+v"(t.idx[c]));
+}
+
+// Every wave computes the same answer (wave-uniform values). Branch-free: the matches
+// of chunk c are a 64-bit ballot; the slots before s are counted, the first three
+// after s extracted.
+__device__ __forceinline__ SlotGroup find_slot_group(const SlotTable& t, int slots, int s,
+                                                     int expert, int E, int lane) {
+    constexpr int kChunks = kGroupMaxSlots / 64;
+    const int sc = s >> 6, sb = s & 63;
+    const uint64_t below = (1ull << sb) - 1ull;
+    uint64_t after[kChunks];
+    int before = 0;
+#pragma unroll
+    for (int c = 0; c < kChunks; c++) {
+        const uint64_t m =
+            __ballot(c * 64 + lane < slots && clamp_expert(t.idx[c], E) == expert);
+        before += __popcll(c < sc ? m : (c == sc ? m & below : 0ull));
+        after[c] = c < sc ? 0ull : (c == sc ? m & ~(below | (1ull << sb)) : m);
+    }
+    int n = 1, next[kGroupRows - 1];
+#pragma unroll
+    for (int take = 0; take < kGroupRows - 1; take++) {
+        int pos = -1;
+#pragma unroll
+        for (int c = kChunks - 1; c >= 0; c--)
+            if (after[c] != 0) pos = c;  // lowest chunk that still has a match
+#pragma unroll
+        for (int c = 0; c < kChunks; c++) {
+            if (pos == c) {
+                pos = c * 64 + (int)__builtin_ctzll(after[c]) + (1 << 20);
+                after[c] &= after[c] - 1;
+            }
+        }
+        next[take] = pos < 0 ? s : pos - (1 << 20);
+        n += pos >= 0;
+    }
+    SlotGroup g;
+    g.expert = expert;
+    g.n = __builtin_amdgcn_readfirstlane((before % kGroupRows) == 0 ? n : 0);
+    g.s0 = s;
+    g.s1 = __builtin_amdgcn_readfirstlane(next[0]);
+    g.s2 = __builtin_amdgcn_readfirstlane(next[1]);
+    g.s3 = __builtin_amdgcn_readfirstlane(next[2]);
+    return g;
+}
+
+__device__ __forceinline__ int group_slot(const SlotGroup& g, int r) {
+    return r == 1 ? g.s1 : (r == 2 ? g.s2 : (r == 3 ? g.s3 : g.s0));
+}
+
+// The NW waves' sums of batch row r, added in wave order.
+template <int NW>
+__device__ __forceinline__ float2_t moe_row_sum(const float (*red)[kGroupRows][128], int r,
+                                                int lane) {
+    float2_t v{red[0][r][2 * lane], red[0][r][2 * lane + 1]};
+#pragma unroll
+    for (int w = 1; w < NW; w++) {
+        v.x = __fadd_rn(v.x, red[w][r][2 * lane]);
+        v.y = __fadd_rn(v.y, red[w][r][2 * lane + 1]);
+    }
+    return v;
+}
+
+// Same grid and arguments as moe_gateup_kernel (+ slots). Wave r of the working
+// workgroup takes batch row r through the split reduction and, as the last
+// contributor of (slot, column block), through gate finish, up finish, GLU and the
+// rotation for the down projection.
+template <int K, int CB, int NW>
+__global__ __launch_bounds__(NW * 64) void moe_gateup_grouped_kernel(
+    const uint32_t* __restrict__ gu_trellis, const half_t* __restrict__ x,
+    const int* __restrict__ indices, const half_t* __restrict__ gu_suh,
+    const half_t* __restrict__ gu_svh, const half_t* __restrict__ dn_suh, half_t* xh_dn,
+    float* part, int* counters, int slots, int top_k, int E, int D, int H, int activation) {
+    __shared__ __attribute__((aligned(16))) half_t xs[NW][kGroupRows][kXwLd];
+    __shared__ float red[NW][kGroupRows][128];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int dblocks = D >> 7, hblocks = H >> 7;
+    const int n_wg = gridDim.y;
+    const int gid = blockIdx.x;
+    const int hg = gid % hblocks, sp = gid / hblocks;
+    const int s = sp >> 1, p = sp & 1;
+    // the first trellis loads only need this slot's own expert: they are in flight
+    // while the routing table is searched; workgroups that carry nothing drop them
+    const int e = clamp_expert(indices[s], E);
+    constexpr bool kHalf = NW == 8;
+    const int part_idx = blockIdx.y * NW + wave;
+    const int blk = kHalf ? part_idx >> 1 : part_idx;
+    // (waves past the last block load the last block's rows and drop them, so that every
+    // wave has the same loads in flight behind the table's)
+    const int tk0 = min(blk, dblocks - 1) * 8 + (kHalf ? (part_idx & 1) * 4 : 0);
+    const int tk1 = tk0 + (kHalf ? 4 : 8);
+    const size_t row_words = (size_t)E * 2 * (H >> 4) * (8 * K);
+    const uint32_t* base =
+        gu_trellis + ((size_t)(p * E + e) * (H >> 4) + 8 * hg) * (8 * K) + lane * K;
+    SlotTable table = load_slot_table(indices, slots, lane);
+    uint32_t buf[kStreamSlots][K];
+    pin_program_order();
+    issue_first_rows<K, kHalf>(opaque_pointer(base), row_words, tk0, tk1, buf);
+    pin_program_order();
+    use_table_from_here(table);
+    const SlotGroup grp = find_slot_group(table, slots, s, e, E, lane);
+    if (grp.n == 0) return;
+    float acc[kGroupRows][2];
+#pragma unroll
+    for (int m = 0; m < kGroupRows; m++) acc[m][0] = acc[m][1] = 0.f;
+    if (blk < dblocks) {
+        const half_t* xrow[kGroupRows];
+#pragma unroll
+        for (int m = 0; m < kGroupRows; m++) xrow[m] = x + (size_t)(group_slot(grp, m) / top_k) * D;
+        stream_block_rows_at<K, CB, kGroupRows, true, kHalf, true, true>(
+            base, row_words, tk0, tk1, xrow, grp.n, gu_suh + ((size_t)e * 2 + p) * D, xs[wave],
+            lane, acc, buf);
+    }
+    const int c0 = (lane >> 3) * 16 + (lane & 7);
+#pragma unroll
+    for (int m = 0; m < kGroupRows; m++) {
+        red[wave][m][c0] = acc[m][0];
+        red[wave][m][c0 + 8] = acc[m][1];
+    }
+    __syncthreads();
+    if (wave >= grp.n) return;
+    const int sr = group_slot(grp, wave);
+    const float2_t v = moe_row_sum<NW>(red, wave, lane);
+    int* counter = counters + sr * hblocks + hg;
+    const size_t gid_r = ((size_t)sr * 2 + p) * hblocks + hg;
+    if (!moe_publish(part + (gid_r * n_wg + blockIdx.y) * 128, v, counter, 2 * n_wg, lane)) return;
+    asm volatile("" ::: "memory");
+    // both projections' partial rows in flight together
+    const float* rows_g = part + (((size_t)sr * 2) * hblocks + hg) * n_wg * 128;
+    const float* rows_u = part + (((size_t)sr * 2 + 1) * hblocks + hg) * n_wg * 128;
+    float2_t sg{0.f, 0.f}, su{0.f, 0.f};
+    for (int i = 0; i < n_wg; i++) {
+        const float2_t fg = __builtin_bit_cast(
+            float2_t, __hip_atomic_load(reinterpret_cast<const uint64_t*>(rows_g + i * 128 + 2 * lane),
+                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        const float2_t fu = __builtin_bit_cast(
+            float2_t, __hip_atomic_load(reinterpret_cast<const uint64_t*>(rows_u + i * 128 + 2 * lane),
+                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        sg.x = __fadd_rn(sg.x, fg.x);
+        sg.y = __fadd_rn(sg.y, fg.y);
+        su.x = __fadd_rn(su.x, fu.x);
+        su.y = __fadd_rn(su.y, fu.y);
+    }
+    const half_t* svh_e = gu_svh + (size_t)e * 2 * H + hg * 128 + 2 * lane;
+    float g0, g1, u0, u1;
+    moe_finish_block(sg, *reinterpret_cast<const half2_t*>(svh_e), lane, g0, g1);
+    moe_finish_block(su, *reinterpret_cast<const half2_t*>(svh_e + H), lane, u0, u1);
+    const float h0 = (float)(half_t)glu_act(g0, u0, activation);
+    const float h1 = (float)(half_t)glu_act(g1, u1, activation);
+    const half2_t ds =
+        *reinterpret_cast<const half2_t*>(dn_suh + (size_t)e * H + hg * 128 + 2 * lane);
+    float a = h0 * (float)ds.x, b = h1 * (float)ds.y;
+    wht128_lanes(a, b, lane);
+    half2_t o;
+    o.x = (half_t)(a * kHadScaleF);
+    o.y = (half_t)(b * kHadScaleF);
+    *reinterpret_cast<half2_t*>(xh_dn + (size_t)sr * H + hg * 128 + 2 * lane) = o;
+    if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Same grid and arguments as moe_down_kernel (+ slots); wave r finishes batch row r.
+template <int K, int CB, int NW>
+__global__ __launch_bounds__(NW * 64) void moe_down_grouped_kernel(
+    const uint32_t* __restrict__ dn_trellis, const half_t* __restrict__ xh_dn,
+    const int* __restrict__ indices, const half_t* __restrict__ dn_svh, half_t* __restrict__ y,
+    float* part, int* counters, int slots, int E, int D, int H) {
+    __shared__ __attribute__((aligned(16))) half_t xs[NW][kGroupRows][kXwLd];
+    __shared__ float red[NW][kGroupRows][128];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int dblocks = D >> 7, hblocks = H >> 7;
+    const int n_wg = gridDim.y;
+    const int gid = blockIdx.x;
+    const int og = gid % dblocks, s = gid / dblocks;
+    const int e = clamp_expert(indices[s], E);
+    constexpr bool kHalf = NW == 8;
+    const int part_idx = blockIdx.y * NW + wave;
+    const int blk = kHalf ? part_idx >> 1 : part_idx;
+    const int tk0 = min(blk, hblocks - 1) * 8 + (kHalf ? (part_idx & 1) * 4 : 0);
+    const int tk1 = tk0 + (kHalf ? 4 : 8);
+    const size_t row_words = (size_t)E * (D >> 4) * (8 * K);
+    const uint32_t* base = dn_trellis + ((size_t)e * (D >> 4) + 8 * og) * (8 * K) + lane * K;
+    SlotTable table = load_slot_table(indices, slots, lane);
+    uint32_t buf[kStreamSlots][K];
+    pin_program_order();
+    issue_first_rows<K, kHalf>(opaque_pointer(base), row_words, tk0, tk1, buf);
+    pin_program_order();
+    use_table_from_here(table);
+    const SlotGroup grp = find_slot_group(table, slots, s, e, E, lane);
+    if (grp.n == 0) return;
+    float acc[kGroupRows][2];
+#pragma unroll
+    for (int m = 0; m < kGroupRows; m++) acc[m][0] = acc[m][1] = 0.f;
+    if (blk < hblocks) {
+        const half_t* xrow[kGroupRows];
+#pragma unroll
+        for (int m = 0; m < kGroupRows; m++) xrow[m] = xh_dn + (size_t)group_slot(grp, m) * H;
+        stream_block_rows_at<K, CB, kGroupRows, false, kHalf, true, true>(
+            base, row_words, tk0, tk1, xrow, grp.n, nullptr, xs[wave], lane, acc, buf);
+    }
+    const int c0 = (lane >> 3) * 16 + (lane & 7);
+#pragma unroll
+    for (int m = 0; m < kGroupRows; m++) {
+        red[wave][m][c0] = acc[m][0];
+        red[wave][m][c0 + 8] = acc[m][1];
+    }
+    __syncthreads();
+    if (wave >= grp.n) return;
+    const int sr = group_slot(grp, wave);
+    float2_t v = moe_row_sum<NW>(red, wave, lane);
+    if (n_wg > 1) {
+        const size_t gid_r = (size_t)sr * dblocks + og;
+        int* counter = counters + gid_r;
+        if (!moe_publish(part + (gid_r * n_wg + blockIdx.y) * 128, v, counter, n_wg, lane)) return;
+        asm volatile("" ::: "memory");
+        v = moe_sum_rows(part + gid_r * n_wg * 128, n_wg, lane);
+        if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    const half2_t sv =
+        *reinterpret_cast<const half2_t*>(dn_svh + (size_t)e * D + og * 128 + 2 * lane);
+    float o0, o1;
+    moe_finish_block(v, sv, lane, o0, o1);
+    half2_t o;
+    o.x = (half_t)o0;
+    o.y = (half_t)o1;
+    *reinterpret_cast<half2_t*>(y + (size_t)sr * D + og * 128 + 2 * lane) = o;
+}
+
 struct MoeWorkspace {
     size_t xh_gu, xh_dn, tables, part_gu, part_dn;
     size_t o_xh_gu, o_xh_dn, o_tables, o_part_gu, o_part_dn, total;
@@ -359,6 +643,13 @@ struct MoeWorkspace {
 static int moe_half_below() {
     static const int v = env_int("EXL3_MOE_HALF_BELOW", 4096, 0, 1 << 20);
     return v;
+}
+
+// Two-launch chain with several tokens: slots of the same expert in one workgroup (1) or
+// every slot on its own (0).
+static bool moe_group_slots() {
+    static const int v = env_int("EXL3_MOE_GROUP", 1, 0, 1);
+    return v != 0;
 }
 
 static MoeWorkspace moe_workspace(int tokens, int top_k, int D, int H) {
@@ -569,8 +860,33 @@ EXL3_EXPORT int exl3_moe_forward(const uint16_t* x, int tokens, const int32_t* i
         // few slots: eight waves per workgroup, each on half a block, so that the
         // chip holds twice the loads in flight (same workgroup count, same partial rows)
         const bool half = (size_t)slots * 2 * hblocks * dblocks < (size_t)moe_half_below();
+        // several tokens: slots of one expert share a pass over its weights, once enough
+        // of them coincide to pay for the table search (from one slot per two experts on:
+        // 16 tokens of top-8 over 256 experts, where ~20 % of the slots share an expert)
+        const bool grouped = tokens > 1 && slots <= kGroupMaxSlots && 2 * slots >= num_experts &&
+                             moe_group_slots();
         auto chain = [&](auto k, auto c, auto nw) {
             constexpr int NW = nw.value;
+            if (grouped) {
+                moe_gateup_grouped_kernel<k.value, c.value, NW>
+                    <<<dim3((unsigned)(slots * 2 * hblocks), (unsigned)((dblocks + 3) / 4)),
+                       dim3(NW * 64), 0, s>>>(reinterpret_cast<const uint32_t*>(gu_trellis),
+                                              reinterpret_cast<const half_t*>(x), indices,
+                                              reinterpret_cast<const half_t*>(gu_suh),
+                                              reinterpret_cast<const half_t*>(gu_svh),
+                                              reinterpret_cast<const half_t*>(dn_suh), xh_dn,
+                                              part_gu, counters, slots, top_k, num_experts, D, H,
+                                              activation);
+                if (int rc = launch_status()) return rc;
+                moe_down_grouped_kernel<k.value, c.value, NW>
+                    <<<dim3((unsigned)(slots * dblocks), (unsigned)((hblocks + 3) / 4)),
+                       dim3(NW * 64), 0, s>>>(reinterpret_cast<const uint32_t*>(dn_trellis), xh_dn,
+                                              indices, reinterpret_cast<const half_t*>(dn_svh),
+                                              reinterpret_cast<half_t*>(y), part_dn,
+                                              counters + (size_t)slots * hblocks, slots,
+                                              num_experts, D, H);
+                return launch_status();
+            }
             moe_gateup_kernel<k.value, c.value, NW>
                 <<<dim3((unsigned)(slots * 2 * hblocks), (unsigned)((dblocks + 3) / 4)),
                    dim3(NW * 64), 0, s>>>(reinterpret_cast<const uint32_t*>(gu_trellis),

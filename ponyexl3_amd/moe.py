@@ -80,19 +80,24 @@ class EXL3SwitchGLU(torch.nn.Module):
             activation=activation,
         )
 
-    # The sorted, segmented prefill path replaces the per-slot kernels once the
-    # experts see about two rows each (the reference switches at 9 tokens,
-    # ponyexl3/mlx/exl3_moe.py:770-787). Measured on 256 experts of 2048 x 512,
-    # top-8: the slot kernels cost ~3.8 us per token (every slot reads its expert),
-    # the prefill path ~0.2 ms whatever the token count (every expert's weights are
-    # decoded once, eight launches); 48 tokens: 181 vs 197 us, 64 tokens: 253 vs
-    # 201 us, so they cross near 56 tokens = 1.75 rows per expert.
+    # The sorted, segmented prefill path replaces the slot kernels once the experts see
+    # a few rows each (the reference switches at 9 tokens,
+    # ponyexl3/mlx/exl3_moe.py:770-787). Measured on 256 experts of 2048 x 512, top-8:
+    # the slot kernels, which share one pass over an expert's weights among up to four
+    # of its slots as long as the call has at most 512 slots, take 64 / 97 / 124 /
+    # 158 us at 16 / 32 / 48 / 64 tokens and 255 us at 72 (576 slots, every slot on
+    # its own); the prefill path takes 180-207 us from 40 to 96 tokens (every expert's
+    # weights are decoded once, eight launches). So: prefill above 512 slots, and
+    # below that from 2.5 rows per expert on (few experts, many rows each).
     prefill_min_tokens = 24
-    prefill_min_rows_per_expert = 1.75
+    prefill_min_rows_per_expert = 2.5
+    grouped_max_slots = 512
 
     def _use_prefill(self, tokens: int, top_k: int) -> bool:
-        return (tokens >= self.prefill_min_tokens
-                and tokens * top_k >= self.prefill_min_rows_per_expert * self.num_experts)
+        slots = tokens * top_k
+        return tokens >= self.prefill_min_tokens and (
+            slots > self.grouped_max_slots
+            or slots >= self.prefill_min_rows_per_expert * self.num_experts)
 
     def forward(self, x: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
         if indices.dim() != 3:

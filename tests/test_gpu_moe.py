@@ -76,6 +76,42 @@ def test_two_launch_and_five_launch_chains(cuda, oracle, tokens):
     assert rel_l2(y1.cpu().numpy(), y5.cpu().numpy()) <= TOL
 
 
+@pytest.mark.parametrize("tokens,top_k,E", [(2, 2, 2), (5, 2, 3), (9, 3, 4), (32, 2, 40), (256, 2, 3)])
+def test_slots_grouped_by_expert_equal_ungrouped(cuda, tokens, top_k, E):
+    """With several tokens the slots of one expert share a pass over its weights, four
+    rows at a time (here up to 171 slots per expert, i.e. many leaders per expert, and
+    the routing table scanned in up to eight chunks). The arithmetic per row is that of
+    the per-slot kernels, so the result is bit-identical to runs that do not group: one
+    token at a time (a token's experts are distinct), and, for the 512-slot case, whose
+    waves take whole Hadamard blocks where a single token's take half blocks, the same
+    tokens inside a 514-slot call, which is past the grouped kernels' routing table."""
+    from ponyexl3_amd import EXL3SwitchGLU, ops
+
+    D, H, k = 384, 256, 4
+    gate, up, down = _experts(E, D, H, k, False, 1300)
+    moe = EXL3SwitchGLU.from_layers(gate, up, down)
+    rng = np.random.default_rng(tokens * 7 + E)
+    x = (rng.standard_normal((tokens + 1, D)) * 0.5).astype(np.float16)
+    idx = np.stack([rng.permutation(E)[:top_k] for _ in range(tokens + 1)]).astype(np.int32)
+    xt, it = torch.from_numpy(x).to(cuda), torch.from_numpy(idx).to(cuda)
+    args = (moe._gu_trellis, moe._gu_suh, moe._gu_svh, moe._dn_trellis, moe._dn_suh, moe._dn_svh, k, moe._cb)
+    print(f"moe grouped tokens={tokens} top_k={top_k} E={E}", flush=True)
+    y = ops.moe_forward(xt[:tokens], it[:tokens], *args)
+    y_again = ops.moe_forward(xt[:tokens], it[:tokens], *args)
+    assert torch.equal(y, y_again)
+    assert int(ops.sync_counters(cuda, 1).abs().sum()) == 0
+    if tokens * top_k == 512:
+        wide = ops.moe_forward(xt, it, *args)
+        assert torch.equal(y, wide[:tokens])
+    step = max(1, tokens // 16)
+    for t in list(range(0, tokens, step)) + [tokens - 1]:
+        one = ops.moe_forward(xt[t:t + 1], it[t:t + 1], *args)
+        if tokens * top_k == 512:
+            assert rel_l2(y[t].float().cpu().numpy(), one[0].float().cpu().numpy()) <= TOL
+        else:
+            assert torch.equal(y[t], one[0]), f"token {t}"
+
+
 @pytest.mark.parametrize("tokens,act", [(40, "silu"), (200, "gelu")])
 def test_prefill_path_matches_oracle_and_slot_kernels(cuda, oracle, tokens, act):
     """From 24 tokens on the pairs are sorted by expert and go through the segmented
