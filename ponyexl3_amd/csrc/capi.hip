@@ -97,7 +97,7 @@ EXL3_EXPORT int exl3_linear_forward(const uint16_t* x, int rows, const uint16_t*
             if (counters_len < linear_small_counter_ints(rows, out_features)) return EXL3_E_WORKSPACE;
             return launch_linear_small(x, rows, trellis, in_tiles, out_tiles, K, cb, suh, n_sub,
                                        group_sub, svh, bias, y, partial, counters,
-                                       plan_linear_small_launch(rows, in_tiles, n_groups), s);
+                                       plan_linear_small_launch(rows, in_tiles, n_groups, K), s);
         }
         if (int rc = launch_had_pre(x, rows, in_features, suh, n_sub, xh, s)) return rc;
         if (int rc = launch_gemv_partials(xh, rows, n_sub, trellis, in_tiles, out_tiles, K, cb,
@@ -249,7 +249,7 @@ EXL3_EXPORT int exl3_linear_forward_static(const uint16_t* x, int rows, const ui
     if (rows > kLinearSmallMaxRows) return EXL3_E_UNSUPPORTED;  // only the one-launch kernel
     if (n_sub > 1 && (!group_sub || !suh)) return EXL3_E_BAD_INDEX;
     const int n_groups = out_tiles / 8;
-    const GemvPlan plan = plan_linear_small_launch(rows, in_tiles, n_groups);
+    const GemvPlan plan = plan_linear_small_launch(rows, in_tiles, n_groups, K);
     const size_t need = exl3_linear_static_need_bytes(rows, in_tiles * 16, out_tiles * 16);
     if (need > kStaticPartialBytes || (size_t)n_groups * sizeof(int32_t) > kStaticCounterBytes)
         return EXL3_E_STATIC_LIMIT;

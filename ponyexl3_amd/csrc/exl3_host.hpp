@@ -61,7 +61,7 @@ struct GemvPlan {
     int n_partials() const { return (n_splits + wg_waves - 1) / wg_waves; }
 };
 GemvPlan plan_gemv(int rows, int in_tiles, int n_groups);
-GemvPlan plan_linear_small(int rows, int in_tiles, int n_groups);
+GemvPlan plan_linear_small(int rows, int in_tiles, int n_groups, int K = 4);
 
 // partial: fp32 [plan.n_partials()][rows][128*n_groups]
 int launch_gemv_partials(const uint16_t* xh, int rows, int n_sub, const uint16_t* trellis,
@@ -80,7 +80,7 @@ constexpr int kLinearSmallMaxRows = kGemvMaxRows;
 bool linear_small_uses_atomics(int rows, int n_groups, GemvPlan plan);
 // plan_linear_small with the reduction in mind: one row on a large layer takes
 // workgroups of eight waves when that brings the launch under the atomics limit.
-GemvPlan plan_linear_small_launch(int rows, int in_tiles, int n_groups);
+GemvPlan plan_linear_small_launch(int rows, int in_tiles, int n_groups, int K = 4);
 inline size_t linear_small_counter_ints(int rows, int out_features) {
     return 2 * (size_t)rows * out_features;  // >= out_features / 128
 }

@@ -464,8 +464,15 @@ GemvPlan plan_gemv(int rows, int in_tiles, int n_groups) {
 
 // Plan of the one-launch layer kernel: splits are whole Hadamard blocks (8 tile
 // rows) and every wave gets the same number of blocks where that divides.
-GemvPlan plan_linear_small(int rows, int in_tiles, int n_groups) {
+GemvPlan plan_linear_small(int rows, int in_tiles, int n_groups, int K) {
     static const int kWavesPerSimd = env_int("EXL3_LINEAR_WAVES_PER_SIMD", 12, 1, 16);
+    // From this K on a wave takes at least two blocks where that still leaves two waves
+    // per SIMD. The kernel holds 7 waves per SIMD up to K = 4, 6 at K = 5..7 and 5 at
+    // K = 8 (VGPRs), so one-block waves come in two to three rounds there; measured at
+    // one row on 5120 -> 34816 / 17408 -> 5120: K = 5 38.4 -> 35.6 / 21.3 -> 21.0 us,
+    // K = 6 43.3 -> 40.1 / 23.5 -> 22.2, K = 8 52.7 -> 47.5 / 29.0 -> 25.4 (K <= 4: no
+    // gain or a loss).
+    static const int kDeepFromK = env_int("EXL3_LINEAR_DEEP_FROM_K", 5, 1, 9);
     // one and two rows: when even one block per wave leaves fewer than this many waves
     // (four per SIMD), the waves take half blocks
     static const int kHalfBelow = env_int("EXL3_LINEAR_HALF_BELOW", 4096, 0, 1 << 20);
@@ -481,6 +488,9 @@ GemvPlan plan_linear_small(int rows, int in_tiles, int n_groups) {
     int blocks_per_split = (n_blocks + max_splits - 1) / max_splits;
     const int n_splits = (n_blocks + blocks_per_split - 1) / blocks_per_split;
     blocks_per_split = (n_blocks + n_splits - 1) / n_splits;
+    if (K >= kDeepFromK && blocks_per_split == 1 && n_blocks >= 2 &&
+        (long long)n_groups * ((n_blocks + 1) / 2) >= 2048)
+        return GemvPlan{(n_blocks + 1) / 2, 16};
     return GemvPlan{n_splits, blocks_per_split * 8};
 }
 
@@ -495,8 +505,8 @@ bool linear_small_uses_atomics(int rows, int n_groups, GemvPlan plan) {
     return (long long)n_groups * plan.n_partials() * 128 * rows <= kMaxAtomics;
 }
 
-GemvPlan plan_linear_small_launch(int rows, int in_tiles, int n_groups) {
-    GemvPlan plan = plan_linear_small(rows, in_tiles, n_groups);
+GemvPlan plan_linear_small_launch(int rows, int in_tiles, int n_groups, int K) {
+    GemvPlan plan = plan_linear_small(rows, in_tiles, n_groups, K);
     if (rows == 1 && plan.tk_per_split >= 8 && !linear_small_uses_atomics(rows, n_groups, plan)) {
         GemvPlan wide = plan;
         wide.wg_waves = 8;
