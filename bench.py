@@ -44,7 +44,7 @@ CB = 0
 # rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE), each scaled
 # by what the same counter reads for a plain copy of known size; see
 # profiles/linear_small_k4_config2_pmc.txt.
-TRAFFIC_BYTES_PER_STEP = 197_827_400
+TRAFFIC_BYTES_PER_STEP = 201_804_400
 
 # (name, in, [member out sizes]) of the config-2 layer; several members = sibling-fused
 LAYER_FUSED_QKV = [
