@@ -316,12 +316,18 @@ int exl3_linear_forward_static(const uint16_t *x, int rows, const uint16_t *trel
  *   activation  0 = silu (SwiGLU), 1 = tanh-gelu (GeGLU) (ponyexl3/mlx/exl3_moe.py:62-75)
  *   y           fp16 [tokens][top_k][D]
  *   workspace   at least exl3_moe_workspace_bytes(tokens, top_k, D, H)
- *   counters    NULL, or int32[counters_len] with counters_len >=
+ *   counters    NULL, or int32[counters_len], 8-byte aligned, with counters_len >=
  *               tokens*top_k*(H/128 + D/128), zero on entry and zero again on
  *               exit. With counters the chain is two launches, the reference's
  *               A2/B2 pair (ponyexl3/mlx/exl3_moe.py:345-422: gate/up, then
  *               GLU + rotation + down); without, five launches that need no
  *               state between calls. Calls that overlap on one counters array race.
+ *               With counters_len >= tokens*top_k*(4*H + D/128) the gate/up launch
+ *               may reduce through 64-bit fixed-point accumulators held there (one
+ *               memory round trip instead of three; chosen when every slot runs on
+ *               its own and the launch issues at most EXL3_MOE_MAX_ATOMICS = 300000
+ *               atomics); the result can differ from the partial-row reduction by
+ *               an fp16 ulp, and is bit-identical from call to call either way.
  * Only the selected experts' trellis blocks are read. In the two-launch chain, with
  * 2 <= tokens, at most 512 slots and at least one slot per two experts, the slots that
  * route to one expert share a pass over its weights (four batch rows per pass; same

@@ -40,7 +40,7 @@ __global__ __launch_bounds__(1024) void diag_decode_kernel(const uint32_t* __res
     constexpr int kSlots = 4;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    xs[threadIdx.x] = (half_t)(float)((threadIdx.x * 37 % 17) - 8);
+    xs[threadIdx.x] = (half_t)(float)((int)(threadIdx.x * 37 % 17) - 8);  // small integers, -8..8
     __syncthreads();
     const uint32_t wave_global = blockIdx.x * 16 + wave;
     float4_t accv[2] = {float4_t{0, 0, 0, 0}, float4_t{0, 0, 0, 0}};

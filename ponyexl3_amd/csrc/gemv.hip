@@ -257,21 +257,6 @@ __global__ __launch_bounds__(NW * 64) void linear_small_kernel(
         const size_t out_total = (size_t)n_groups * 128;
         const int wg_splits = (n_splits + NW - 1) / NW;  // partial rows per group
         const size_t col = (size_t)g * 128 + 2 * lane;
-        constexpr float kFixScale = 16777216.f;         // 2^24
-        constexpr float kFixClamp = 262144.f;           // |partial| is clamped to 2^18 (fp16 ends at 65504)
-        auto to_word = [&](float v) -> unsigned long long {
-            v = fminf(fmaxf(v, -kFixClamp), kFixClamp);
-            const long long fixed = (long long)((double)v * (double)kFixScale);
-            return (1ull << 56) + (unsigned long long)fixed;
-        };
-        auto word_count = [](unsigned long long w) -> int {
-            return (int)((long long)(w + (1ull << 55)) >> 56);
-        };
-        auto word_value = [&](unsigned long long w) -> float {
-            const long long c = (long long)(w + (1ull << 55)) >> 56;
-            const long long fixed = (long long)(w - ((unsigned long long)c << 56));
-            return (float)((double)fixed * (1.0 / (double)kFixScale));
-        };
         unsigned long long w0[MT], w1[MT];
 #pragma unroll
         for (int m = 0; m < MT; m++) {
@@ -283,20 +268,20 @@ __global__ __launch_bounds__(NW * 64) void linear_small_kernel(
                     vx = __fadd_rn(vx, red[w][m][2 * lane]);
                     vy = __fadd_rn(vy, red[w][m][2 * lane + 1]);
                 }
-                const unsigned long long ax = to_word(vx), ay = to_word(vy);
+                const unsigned long long ax = fix_word(vx), ay = fix_word(vy);
                 unsigned long long* slot = sums + (size_t)m * out_total + col;
                 w0[m] = __hip_atomic_fetch_add(slot, ax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + ax;
                 w1[m] = __hip_atomic_fetch_add(slot + 1, ay, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + ay;
             }
         }
         // lane 0's first word is (row 0, first column of the group)
-        const int first_count = __builtin_amdgcn_readfirstlane(word_count(w0[0]));
+        const int first_count = __builtin_amdgcn_readfirstlane(fix_count(w0[0]));
         if (first_count != wg_splits) return;
         auto all_complete = [&]() {
             bool ok = true;
 #pragma unroll
             for (int m = 0; m < MT; m++)
-                if (m < rows) ok = ok && word_count(w0[m]) == wg_splits && word_count(w1[m]) == wg_splits;
+                if (m < rows) ok = ok && fix_count(w0[m]) == wg_splits && fix_count(w1[m]) == wg_splits;
             return __ballot(ok) == ~0ull;
         };
         for (int spin = 0; !all_complete() && spin < (1 << 22); spin++) {
@@ -320,8 +305,8 @@ __global__ __launch_bounds__(NW * 64) void linear_small_kernel(
                 __hip_atomic_store(slot + 1, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 // the cast at ponyexl3/ref/forward.py:41, then the output Hadamard of this one
                 // 128-column block, svh and bias (forward.py:42-45)
-                float a = (float)(half_t)word_value(w0[m]);
-                float b = (float)(half_t)word_value(w1[m]);
+                float a = (float)(half_t)fix_value(w0[m]);
+                float b = (float)(half_t)fix_value(w1[m]);
                 wht128_lanes(a, b, lane);
                 a = __fmul_rn(a, kHadScaleF);
                 b = __fmul_rn(b, kHadScaleF);

@@ -294,6 +294,96 @@ __global__ __launch_bounds__(NW * 64) void moe_gateup_kernel(
     if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Gate and up of one k-chunk in ONE workgroup of eight waves, reduced through 64-bit
+// accumulators with returning atomics (see fix_word): waves 0..3 stream gate, waves
+// 4..7 up, over the same Hadamard blocks of D - HALF: half a block each, two blocks
+// per workgroup; else a block each, four blocks per workgroup. Wave 0 adds the
+// workgroup's 128 gate sums and 128 up sums to the accumulators of (slot, column
+// block); the workgroup whose add completes the first gate column is the finisher: it
+// holds (or polls for, if other workgroups' adds were interleaved with its own) both
+// totals, so it goes on to post-Hadamard, svh, GLU and the rotation for the down
+// projection without another trip through memory. One round trip instead of the
+// three of store / counter / reload.
+// grid = (slots * H/128, chunks); sums: uint64 [slots][2][H], zero on entry and exit.
+template <int K, int CB, bool HALF>
+__global__ __launch_bounds__(512) void moe_gateup_pair_kernel(
+    const uint32_t* __restrict__ gu_trellis, const half_t* __restrict__ x,
+    const int* __restrict__ indices, const half_t* __restrict__ gu_suh,
+    const half_t* __restrict__ gu_svh, const half_t* __restrict__ dn_suh, half_t* xh_dn,
+    unsigned long long* sums, int top_k, int E, int D, int H, int activation) {
+    __shared__ __attribute__((aligned(16))) half_t xs[8][1][kXwLd];
+    __shared__ float red[8][128];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int dblocks = D >> 7, hblocks = H >> 7;
+    const int n_chunks = gridDim.y;
+    const int gid = blockIdx.x;
+    const int hg = gid % hblocks, s = gid / hblocks;
+    const int p = wave >> 2, j = wave & 3;
+    const int e = clamp_expert(indices[s], E);
+    const int blk = HALF ? blockIdx.y * 2 + (j >> 1) : blockIdx.y * 4 + j;
+    const int tk0 = blk * 8 + (HALF ? (j & 1) * 4 : 0);
+    float acc[1][2] = {{0.f, 0.f}};
+    if (blk < dblocks) {
+        const size_t row_words = (size_t)E * 2 * (H >> 4) * (8 * K);
+        const uint32_t* base =
+            gu_trellis + ((size_t)(p * E + e) * (H >> 4) + 8 * hg) * (8 * K) + lane * K;
+        stream_block_rows<K, CB, 1, true, HALF>(base, row_words, tk0, tk0 + (HALF ? 4 : 8),
+                                                x + (size_t)(s / top_k) * D, (size_t)D, 1,
+                                                gu_suh + ((size_t)e * 2 + p) * D, xs[wave], lane,
+                                                acc);
+    }
+    const int c0 = (lane >> 3) * 16 + (lane & 7);
+    red[wave][c0] = acc[0][0];
+    red[wave][c0 + 8] = acc[0][1];
+    __syncthreads();
+    if (wave != 0) return;
+    // word q of a lane: projection q >> 1, column 2*lane + (q & 1); wave order within a projection
+    unsigned long long w[4];
+    unsigned long long* slot[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int col = 2 * lane + (q & 1), w0 = (q >> 1) * 4;
+        float v = red[w0][col];
+#pragma unroll
+        for (int i = 1; i < 4; i++) v = __fadd_rn(v, red[w0 + i][col]);
+        slot[q] = sums + ((size_t)s * 2 + (q >> 1)) * H + hg * 128 + col;
+        const unsigned long long a = fix_word(v);
+        w[q] = __hip_atomic_fetch_add(slot[q], a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + a;
+    }
+    if (__builtin_amdgcn_readfirstlane(fix_count(w[0])) != n_chunks) return;
+    auto all_complete = [&]() {
+        bool ok = true;
+#pragma unroll
+        for (int q = 0; q < 4; q++) ok = ok && fix_count(w[q]) == n_chunks;
+        return __ballot(ok) == ~0ull;
+    };
+    for (int spin = 0; !all_complete() && spin < (1 << 22); spin++) {
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+            w[q] = __hip_atomic_load(slot[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+        __hip_atomic_store(slot[q], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const half_t* svh_e = gu_svh + (size_t)e * 2 * H + hg * 128 + 2 * lane;
+    float g0, g1, u0, u1;
+    moe_finish_block(float2_t{fix_value(w[0]), fix_value(w[1])},
+                     *reinterpret_cast<const half2_t*>(svh_e), lane, g0, g1);
+    moe_finish_block(float2_t{fix_value(w[2]), fix_value(w[3])},
+                     *reinterpret_cast<const half2_t*>(svh_e + H), lane, u0, u1);
+    const float h0 = (float)(half_t)glu_act(g0, u0, activation);
+    const float h1 = (float)(half_t)glu_act(g1, u1, activation);
+    const half2_t ds =
+        *reinterpret_cast<const half2_t*>(dn_suh + (size_t)e * H + hg * 128 + 2 * lane);
+    float a = h0 * (float)ds.x, b = h1 * (float)ds.y;
+    wht128_lanes(a, b, lane);
+    half2_t o;
+    o.x = (half_t)(a * kHadScaleF);
+    o.y = (half_t)(b * kHadScaleF);
+    *reinterpret_cast<half2_t*>(xh_dn + (size_t)s * H + hg * 128 + 2 * lane) = o;
+}
+
 // grid = (slots * D/128, ceil((H/128) / 4)); slot s = gid / dblocks, column block
 // og = gid % dblocks. xh_dn is already rotated. part: fp32 [gid][n_wg][128].
 template <int K, int CB, int NW>
@@ -652,6 +742,13 @@ static bool moe_group_slots() {
     return v != 0;
 }
 
+// Gate/up launches that would issue more atomics than this reduce through partial rows
+// (the memory side retires about 75 000 returning atomics per microsecond).
+static long long moe_max_atomics() {
+    static const int v = env_int("EXL3_MOE_MAX_ATOMICS", 300000, 0, 1 << 30);
+    return v;
+}
+
 static MoeWorkspace moe_workspace(int tokens, int top_k, int D, int H) {
     MoeWorkspace w{};
     const int slots = tokens * top_k;
@@ -865,8 +962,36 @@ EXL3_EXPORT int exl3_moe_forward(const uint16_t* x, int tokens, const int32_t* i
         // 16 tokens of top-8 over 256 experts, where ~20 % of the slots share an expert)
         const bool grouped = tokens > 1 && slots <= kGroupMaxSlots && 2 * slots >= num_experts &&
                              moe_group_slots();
+        // every slot on its own, few enough atomics, and counters large enough to hold
+        // the accumulators (uint64 [slots][2][H], then the down launch's counters): gate
+        // and up of a k-chunk in one workgroup, reduced through returning atomics
+        const int pair_chunks = half ? (dblocks + 1) / 2 : (dblocks + 3) / 4;
+        const size_t pair_ints = (size_t)slots * 2 * H * 2;
+        const bool pair = !grouped && pair_chunks <= 255 &&
+                          (long long)slots * 2 * H * pair_chunks <= moe_max_atomics() &&
+                          counters_len >= pair_ints + (size_t)slots * dblocks &&
+                          (reinterpret_cast<uintptr_t>(counters) & 7) == 0;
         auto chain = [&](auto k, auto c, auto nw) {
             constexpr int NW = nw.value;
+            if (pair) {
+                moe_gateup_pair_kernel<k.value, c.value, NW == 8>
+                    <<<dim3((unsigned)(slots * hblocks), (unsigned)pair_chunks), dim3(512), 0, s>>>(
+                        reinterpret_cast<const uint32_t*>(gu_trellis),
+                        reinterpret_cast<const half_t*>(x), indices,
+                        reinterpret_cast<const half_t*>(gu_suh),
+                        reinterpret_cast<const half_t*>(gu_svh),
+                        reinterpret_cast<const half_t*>(dn_suh), xh_dn,
+                        reinterpret_cast<unsigned long long*>(counters), top_k, num_experts, D, H,
+                        activation);
+                if (int rc = launch_status()) return rc;
+                moe_down_kernel<k.value, c.value, NW>
+                    <<<dim3((unsigned)(slots * dblocks), (unsigned)((hblocks + 3) / 4)),
+                       dim3(NW * 64), 0, s>>>(reinterpret_cast<const uint32_t*>(dn_trellis), xh_dn,
+                                              indices, reinterpret_cast<const half_t*>(dn_svh),
+                                              reinterpret_cast<half_t*>(y), part_dn,
+                                              counters + pair_ints, num_experts, D, H);
+                return launch_status();
+            }
             if (grouped) {
                 moe_gateup_grouped_kernel<k.value, c.value, NW>
                     <<<dim3((unsigned)(slots * 2 * hblocks), (unsigned)((dblocks + 3) / 4)),

@@ -641,10 +641,12 @@ def linear_forward(x2d, trellis, k, cb, suh=None, svh=None, bias=None, group_sub
 
 
 def moe_forward(x2d, indices, gu_trellis, gu_suh, gu_svh, dn_trellis, dn_suh, dn_svh, k, cb,
-                activation: int = 0, fused: bool = True):
+                activation: int = 0, fused: bool = True, accumulators: bool = True):
     """(T, D) fp16, (T, top_k) int32 -> (T, top_k, D) fp16 (``exl3_moe_forward``).
-    ``fused`` selects the two-launch chain (needs the per-device counters);
-    otherwise the five-launch chain runs."""
+    ``fused`` selects the two-launch chain (needs the per-stream counters);
+    otherwise the five-launch chain runs. ``accumulators`` hands the library enough
+    counter memory for the gate/up reduction through 64-bit accumulators (it then
+    chooses per call); without, the reduction goes through partial rows."""
     _half(x2d, "x")
     _check_cuda(indices, "indices")
     if indices.dtype != torch.int32 or indices.dim() != 2:
@@ -659,13 +661,13 @@ def moe_forward(x2d, indices, gu_trellis, gu_suh, gu_svh, dn_trellis, dn_suh, dn
     if ws_bytes == 0:
         raise ValueError("MoE dims must be positive multiples of 128")
     ws = workspace(x2d.device, ws_bytes)
-    n_cnt = T * top_k * (D // 128 + H // 128)
+    n_cnt = T * top_k * ((4 * H if accumulators else H // 128) + D // 128)
     cnt = sync_counters(x2d.device, n_cnt) if fused else None
     rc = lib.exl3_moe_forward(
         _ptr(x2d), T, _ptr(indices), top_k, _ptr(gu_trellis), _ptr(gu_suh), _ptr(gu_svh),
         _ptr(dn_trellis), _ptr(dn_suh), _ptr(dn_svh), E, D, H, int(k), int(cb), int(activation),
         _ptr(y), _ptr(ws), ws.numel(), _ptr(cnt) if cnt is not None else None,
-        cnt.numel() if cnt is not None else 0, _stream(),
+        n_cnt if cnt is not None else 0, _stream(),  # the length asked for, not the buffer's
     )
     _lib.check(rc, "exl3_moe_forward")
     return y

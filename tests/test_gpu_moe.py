@@ -100,16 +100,55 @@ def test_slots_grouped_by_expert_equal_ungrouped(cuda, tokens, top_k, E):
     y_again = ops.moe_forward(xt[:tokens], it[:tokens], *args)
     assert torch.equal(y, y_again)
     assert int(ops.sync_counters(cuda, 1).abs().sum()) == 0
+    # the runs that do not group reduce through partial rows like the grouped kernels
+    # (accumulators=False); the accumulator reduction rounds the sum differently
     if tokens * top_k == 512:
-        wide = ops.moe_forward(xt, it, *args)
+        wide = ops.moe_forward(xt, it, *args, accumulators=False)
         assert torch.equal(y, wide[:tokens])
     step = max(1, tokens // 16)
     for t in list(range(0, tokens, step)) + [tokens - 1]:
-        one = ops.moe_forward(xt[t:t + 1], it[t:t + 1], *args)
+        one = ops.moe_forward(xt[t:t + 1], it[t:t + 1], *args, accumulators=False)
         if tokens * top_k == 512:
             assert rel_l2(y[t].float().cpu().numpy(), one[0].float().cpu().numpy()) <= TOL
         else:
             assert torch.equal(y[t], one[0]), f"token {t}"
+
+
+@pytest.mark.parametrize("tokens,top_k,E,D,H,act", [(1, 2, 4, 640, 640, 0), (1, 8, 64, 2048, 512, 0),
+                                                     (3, 2, 64, 384, 256, 1), (8, 8, 256, 512, 256, 0)])
+def test_accumulator_reduction_of_gate_up(cuda, oracle, tokens, top_k, E, D, H, act):
+    """Every slot on its own: gate and up of a k-chunk run in one workgroup and meet the
+    other chunks in 64-bit accumulators (D of five blocks: three chunks of two blocks, the
+    last half empty; 16 blocks: eight chunks). Against the partial-row reduction of the
+    same call (an fp16 ulp at most: same products, the sum rounded once instead of per
+    row), twice in a row bit for bit, with the accumulators back at zero."""
+    from ponyexl3_amd import EXL3SwitchGLU, ops
+
+    k = 4
+    rng = np.random.default_rng(tokens * 31 + E)
+    if E <= 8:
+        gate, up, down = _experts(E, D, H, k, False, 1500)
+        moe = EXL3SwitchGLU.from_layers(gate, up, down, activation="silu" if act == 0 else "gelu")
+    else:  # random stacks: many experts without building them one by one
+        rnd = lambda *s: torch.from_numpy(rng.integers(-32768, 32768, size=s, dtype=np.int16)).to(cuda)
+        sgn = lambda *s: torch.from_numpy(np.where(rng.random(s) > 0.5, -1.0, 1.0).astype(np.float16)).to(cuda)
+        moe = EXL3SwitchGLU(gu_trellis=rnd(D // 16, E * 2 * H // 16, 16 * k), gu_suh=sgn(E, 2, D),
+                            gu_svh=sgn(E, 2 * H), dn_trellis=rnd(H // 16, E * D // 16, 16 * k),
+                            dn_suh=sgn(E, H), dn_svh=sgn(E, D), k=k, cb=0)
+    x = torch.from_numpy((rng.standard_normal((tokens, D)) * 0.25).astype(np.float16)).to(cuda)
+    idx = torch.from_numpy(np.stack([rng.permutation(E)[:top_k] for _ in range(tokens)]).astype(np.int32)).to(cuda)
+    args = (x, idx, moe._gu_trellis, moe._gu_suh, moe._gu_svh, moe._dn_trellis, moe._dn_suh, moe._dn_svh, k,
+            moe._cb, act)
+    print(f"moe accumulators tokens={tokens} top_k={top_k} E={E} D={D} H={H}", flush=True)
+    ya = ops.moe_forward(*args)
+    ya2 = ops.moe_forward(*args)
+    yp = ops.moe_forward(*args, accumulators=False)
+    assert torch.equal(ya, ya2)
+    assert int(ops.sync_counters(cuda, 1).abs().sum()) == 0
+    assert rel_l2(ya.float().cpu().numpy(), yp.float().cpu().numpy()) <= 5e-4  # fp16 ulps over three casts
+    if E <= 8:
+        ref = _oracle_chain(oracle, gate, up, down, x.cpu().numpy(), idx.cpu().numpy(), "silu" if act == 0 else "gelu")
+        assert rel_l2(ya.cpu().numpy(), ref) <= TOL
 
 
 @pytest.mark.parametrize("tokens,act", [(40, "silu"), (200, "gelu")])
