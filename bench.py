@@ -461,6 +461,24 @@ def bench_ceilings(dev):
         torch.cuda.synchronize()
         return a.elapsed_time(b) / len(launches)
 
+    def timed_graph(launches):
+        """mean ms per launch of the thunks captured into one HIP graph and replayed"""
+        for fn in launches:
+            fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for fn in launches:
+                fn()
+        g.replay()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / len(launches)
+
     chunk = 512 << 20
     read = [(lambda o=o: _lib.check(lib.exl3_diag_stream_read(ptr(o), chunk, ctypes.c_void_p(out.data_ptr()), stream()),
                                     "exl3_diag_stream_read")) for o in range(0, total, chunk)]
@@ -486,6 +504,25 @@ def bench_ceilings(dev):
     res["decode_loop"] = loops
     res["decode_loop_note"] = ("n_cu workgroups x 16 waves x 128 tile rows per launch, launch overhead included "
                                "(about 10 % of a launch)")
+    # The phases of a layer-kernel launch that no decoding overlaps, on the four grids of
+    # the timed step (K=4, one row): dispatch of the grid alone, and dispatch + every
+    # wave's first four tile rows arriving from cold memory.
+    phases = {}
+    n_rows = total // (256 * K_BITS)
+    for name, gx, gy, threads in (("qkv_proj", 80, 20, 256), ("o_proj", 40, 16, 256),
+                                  ("gate_up", 272, 5, 512), ("down_proj", 40, 34, 256)):
+        waves = gx * gy * threads // 64
+        empty = [(lambda: _lib.check(lib.exl3_diag_empty_launch(gx, gy, threads, stream()),
+                                     "exl3_diag_empty_launch"))] * 64
+        stride = max(waves * 4, n_rows // 64)
+        first = [(lambda i=i: _lib.check(lib.exl3_diag_first_rows(ptr(0), total, K_BITS, gx, gy, threads,
+                                                                   (i * stride) % n_rows,
+                                                                   ctypes.c_void_p(out.data_ptr()), stream()),
+                                         "exl3_diag_first_rows")) for i in range(64)]
+        phases[name] = {"grid": f"{gx}x{gy}x{threads}", "dispatch_us": round(timed_graph(empty) * 1e3, 2),
+                        "dispatch_and_first_rows_us": round(timed_graph(first) * 1e3, 2)}
+    res["launch_phases"] = phases
+    res["launch_phases_note"] = "64 launches back to back inside one HIP graph (device-side rate, no host launch cost)"
     del buf, out
     return res
 

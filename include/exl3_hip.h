@@ -58,10 +58,20 @@ const char *exl3_status_string(int status);
  *   consecutive 256*K-byte rows of buf, wrapping at the largest power-of-two row
  *   count that fits in `bytes`; weights per launch = n_wg*16*steps*2048. cb 0 or 1.
  *   out: float [n_wg*1024].
+ * exl3_diag_empty_launch: a kernel that does nothing on a grid of grid_x * grid_y
+ *   workgroups of `threads` lanes (a multiple of 64, at most 1024): what the dispatch of
+ *   such a grid costs.
+ * exl3_diag_first_rows: on the same kind of grid every wave requests its first four
+ *   tile rows (wave-wide loads of 256*K bytes, rows row_base + 4*wave .. +3 of buf,
+ *   wrapping like above), waits for them and leaves: the time before a small-batch
+ *   launch can decode anything. out: 4 bytes of device memory, practically never written.
  */
 int exl3_diag_stream_read(const void *buf, size_t bytes, void *out, void *stream);
 int exl3_diag_decode_loop(const void *buf, size_t bytes, int K, int cb, int n_wg, int steps,
                           float *out, void *stream);
+int exl3_diag_empty_launch(int grid_x, int grid_y, int threads, void *stream);
+int exl3_diag_first_rows(const void *buf, size_t bytes, int K, int grid_x, int grid_y,
+                         int threads, unsigned row_base, void *out, void *stream);
 
 /* Largest row count the small-batch kernel (exl3_gemv) accepts per call. */
 int exl3_gemv_max_rows(void);

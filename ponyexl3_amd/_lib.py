@@ -34,6 +34,8 @@ PROTOTYPES = {
     "exl3_status_string": (ctypes.c_char_p, [_i]),
     "exl3_diag_stream_read": (_i, [_vp, _sz, _vp, _vp]),
     "exl3_diag_decode_loop": (_i, [_vp, _sz, _i, _i, _i, _i, _vp, _vp]),
+    "exl3_diag_empty_launch": (_i, [_i, _i, _i, _vp]),
+    "exl3_diag_first_rows": (_i, [_vp, _sz, _i, _i, _i, _i, ctypes.c_uint, _vp, _vp]),
     "exl3_gemv_max_rows": (_i, []),
     "exl3_linear_small_max_rows": (_i, []),
     "exl3_decode_full": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _vp]),

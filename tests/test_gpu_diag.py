@@ -51,3 +51,21 @@ def test_decode_loop(cuda, k, cb):
     assert bad(nbytes=16) == _lib.EXL3_E_BAD_SHAPE
     assert bad(cb=2) == _lib.EXL3_E_UNSUPPORTED
     assert bad(k=9) != 0
+
+
+def test_launch_phase_probes(cuda):
+    _lib, lib, buf, stream = _args(cuda)
+    out = torch.zeros(4, dtype=torch.int32, device=cuda)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    print("diag launch phases", flush=True)
+    assert lib.exl3_diag_empty_launch(40, 16, 256, stream) == 0
+    assert lib.exl3_diag_empty_launch(272, 5, 512, stream) == 0
+    for k in (2, 4, 5, 8):
+        assert lib.exl3_diag_first_rows(p(buf), buf.numel() * 4, k, 40, 16, 256, 12345, p(out), stream) == 0
+    torch.cuda.synchronize()
+    assert lib.exl3_diag_empty_launch(0, 1, 256, stream) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_diag_empty_launch(4, 1, 100, stream) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_diag_empty_launch(4, 1, 2048, stream) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_diag_first_rows(None, 4096, 4, 4, 1, 256, 0, p(out), stream) == _lib.EXL3_E_NULL_POINTER
+    assert lib.exl3_diag_first_rows(p(buf), 100, 4, 4, 1, 256, 0, p(out), stream) == _lib.EXL3_E_BAD_SHAPE
+    assert lib.exl3_diag_first_rows(p(buf), buf.numel() * 4, 9, 4, 1, 256, 0, p(out), stream) != 0
