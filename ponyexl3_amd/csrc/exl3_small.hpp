@@ -193,10 +193,14 @@ __device__ __forceinline__ void stream_block_rows_at(const uint32_t* __restrict_
         }
     };
     constexpr int kSlots = kStreamSlots;
+    // The activations are requested before the trellis rows: loads return in issue
+    // order, so the rotation then only waits for the activations and the decode of the
+    // first row only for that row, not for all kSlots rows.
+    fetch_block(tk_begin >> 3);
     if constexpr (!PRELOADED) issue_first_rows<K, HALF>(base, row_words, tk_begin, tk_end, buf);
+    __builtin_amdgcn_sched_barrier(0);  // all of them in flight before the rotation starts
     if constexpr (HALF) {
         // all four loads up front, no refills
-        fetch_block(tk_begin >> 3);
         stage_block();
         const int row0 = tk_begin & 7;  // 0 or 4
         uint32_t prev = neighbour_word(buf[0][K - 1], lane);
@@ -219,10 +223,12 @@ __device__ __forceinline__ void stream_block_rows_at(const uint32_t* __restrict_
     }
     // Ranges are whole blocks, so the staging sits outside the unrolled 8-step
     // pipeline and the LDS offsets of the activations are compile-time constants.
-    fetch_block(tk_begin >> 3);
+    // (the first block is staged before anything touches the trellis rows)
+    stage_block();
     uint32_t prev = neighbour_word(buf[0][K - 1], lane);
-    for (int tkb = tk_begin; tkb < tk_end; tkb += 8) {
-        stage_block();
+    int tkb = tk_begin;
+    do {  // the range is not empty (no loop guard for loads to sink behind)
+        if (tkb != tk_begin) stage_block();
         if (tkb + 8 < tk_end) fetch_block((tkb >> 3) + 1);
 #pragma unroll
         for (int s8 = 0; s8 < 8; s8++) {
@@ -237,7 +243,8 @@ __device__ __forceinline__ void stream_block_rows_at(const uint32_t* __restrict_
             __builtin_amdgcn_sched_barrier(0);
             prev = prev_next;
         }
-    }
+        tkb += 8;
+    } while (tkb < tk_end);
 #pragma unroll
     for (int m = 0; m < MT; m++) {
         acc[m][0] += accv[0][m >> 2][m & 3];
