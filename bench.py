@@ -44,7 +44,7 @@ CB = 0
 # rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE), each scaled
 # by what the same counter reads for a plain copy of known size; see
 # profiles/linear_small_k4_config2_pmc.txt.
-TRAFFIC_BYTES_PER_STEP = 201_804_400
+TRAFFIC_BYTES_PER_STEP = 201_456_400
 
 # (name, in, [member out sizes]) of the config-2 layer; several members = sibling-fused
 LAYER_FUSED_QKV = [
@@ -264,25 +264,35 @@ def main():
     torch.cuda.synchronize()
     # exactly --steps steps between two synchronisations, --repeats times; the
     # reported figure is the median of the repeats (a 20-step region is under 2 ms)
-    samples = []
+    samples, event_samples = [], []
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     for _ in range(max(1, args.repeats)):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
+        ev0.record()  # HIP events on the stream the kernels are launched on
         run_steps(args.steps)
+        ev1.record()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
         samples.append((t1 - t0) * 1e3 / args.steps)
+        event_samples.append(ev0.elapsed_time(ev1) / args.steps)
     ms_per_step = float(np.median(samples))
+    event_ms_per_step = float(np.median(event_samples))
     value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
 
     # ---- roofline of the dominant kernel: the one-launch layer kernel (input
-    # Hadamard + decode GEMV + split reduction + output Hadamard). Its launch
-    # duration is measured per linear with two HIP events around back-to-back
-    # graph replays; a graph holds one launch per weight copy, with enough seeded
-    # copies of that linear (>= 320 MB) that no launch finds its weights in the
-    # 256 MB last-level cache. Durations measured this way agree with rocprofv3's
-    # per-dispatch figures to about a microsecond (the gap between dependent
-    # launches), see profiles/.
+    # Hadamard + decode GEMV + split reduction + output Hadamard). The timed step is
+    # four launches of it and nothing else, so its average launch duration over the
+    # timed region is the HIP-event time of the region / (4 * steps), and achieved =
+    # weight bytes of a step / event time of a step. rocprofv3's per-dispatch durations
+    # of the same four launches add up to the same figure (profiles/).
+    # per_linear: each launch shape on its own, two HIP events around back-to-back
+    # replays of a graph that holds at least 32 launches walking over enough seeded
+    # copies of that linear (>= 320 MB) that no launch finds its weights in the 256 MB
+    # last-level cache. In such a run of identical launches gate+up takes about 4 us
+    # longer than inside the step (34.7 vs 30.2 us median by a kernel trace of the same
+    # process; the other three shapes 0.1-0.6 us), so the sum of the per_linear figures
+    # is above the step time.
     per_linear = {}
     tot_bytes = tot_ms = 0.0
     for j, (name, n_in, outs) in enumerate(LAYER):
@@ -292,7 +302,8 @@ def main():
                             "GBps": round(nb / ms / 1e6, 1)}
         tot_bytes += nb
         tot_ms += ms
-    achieved = tot_bytes / tot_ms / 1e6
+    isolated = tot_bytes / tot_ms / 1e6
+    achieved = bytes_per_step / event_ms_per_step / 1e6
     roofline = {
         "bound": "hbm",
         "kernel": "linear_small_kernel<K=4, cb=3INST, rows=1>",
@@ -303,9 +314,16 @@ def main():
         "traffic": TRAFFIC_BYTES_PER_STEP,
         "traffic_source": "profiles/linear_small_k4_config2_pmc.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this "
                           "script, scaled by a 64 MiB copy); a constant, not measured in this run",
-        "bytes_per_launch": "in*out*K/8 of the launch's linear(s); achieved = sum over the launches of a step / "
-                            "sum of their mean durations; traffic = HBM bytes of the same launches (FETCH_SIZE + WRITE_SIZE)",
+        "bytes_per_launch": "in*out*K/8 of the launch's linear(s): 45.2 MB on average over the four launches of a "
+                            "step; achieved = weight bytes of a step / HIP-event time of a step over the timed region "
+                            "(= bytes per launch / average launch duration); traffic = HBM bytes of the same four "
+                            "launches (FETCH_SIZE + WRITE_SIZE)",
+        "avg_launch_us": round(event_ms_per_step * 1e3 / len(LAYER), 2),
+        "event_ms_per_step": round(event_ms_per_step, 5),
         "per_linear": per_linear,
+        "per_linear_note": "each launch shape replayed on its own (>= 32 identical launches per graph, cold weights); "
+                           "gate_up runs about 4 us longer that way than inside the step",
+        "achieved_from_per_linear": round(isolated, 1),
     }
 
     ceilings = bench_ceilings(dev)
@@ -375,8 +393,11 @@ def _time_ms(fn, reps, warm=3):
 
 def _launch_ms(lin, x, k, dev, cb=CB, min_bytes=320e6, reps=20):
     """Mean duration of one layer-kernel launch of the linear `lin` (its shape,
-    signs and sibling table) with K = k on cold weights: one graph of one launch
-    per seeded weight copy, replayed back to back between two HIP events."""
+    signs and sibling table) with K = k on cold weights: one graph that walks over
+    the seeded weight copies (>= min_bytes in all, so that no launch finds its
+    weights in the last-level cache) often enough to hold at least 32 launches (the
+    cost of replaying a graph is then a small share of a launch), replayed back to
+    back between two HIP events."""
     import torch
 
     from ponyexl3_amd import ops
@@ -392,10 +413,11 @@ def _launch_ms(lin, x, k, dev, cb=CB, min_bytes=320e6, reps=20):
     for tr in trs:
         call(tr)
     torch.cuda.synchronize()
+    cycles = max(1, int(np.ceil(32 / copies)))
     gr = torch.cuda.CUDAGraph()
     with torch.cuda.graph(gr):
-        keep = [call(tr) for tr in trs]
-    ms = _time_batch_ms(gr.replay, reps=reps, warm=3) / copies
+        keep = [call(tr) for _ in range(cycles) for tr in trs]
+    ms = _time_batch_ms(gr.replay, reps=max(4, reps // cycles), warm=3) / (copies * cycles)
     del gr, keep, trs
     return ms
 
