@@ -298,8 +298,10 @@ size_t exl3_linear_workspace_bytes(int rows, int in_features, int out_features, 
  * library runs on holds its copy until the process ends. No hipMalloc, hipFree or
  * other allocating call is made.
  *   rows <= exl3_gemv_max_rows(), otherwise EXL3_E_UNSUPPORTED;
- *   exl3_linear_static_need_bytes(rows, in, out) must not exceed the scratch size,
- *   otherwise EXL3_E_STATIC_LIMIT (nothing is launched).
+ *   exl3_linear_static_need_bytes(rows, in, out) (the largest of what the launch
+ *   plans of the different K keep in either half) must not exceed the scratch size;
+ *   a launch whose own plan needs more returns EXL3_E_STATIC_LIMIT (nothing is
+ *   launched).
  * All calls on one GPU share that GPU's array: calls that overlap there (two
  * streams, two threads) race. The counter half is all zero whenever no call is
  * running.

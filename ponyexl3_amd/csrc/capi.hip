@@ -227,13 +227,35 @@ static int static_scratch(hipStream_t stream, unsigned char** out) {
 
 EXL3_EXPORT size_t exl3_linear_static_scratch_bytes(void) { return exl3::kStaticPartialBytes; }
 
+namespace exl3 {
+
+// What a launch with this plan keeps in the two halves of the array: fp32 partial rows
+// and group counters, or the accumulators (which live in the counter half).
+struct StaticNeed {
+    size_t partial_bytes, counter_bytes;
+    size_t larger() const { return partial_bytes > counter_bytes ? partial_bytes : counter_bytes; }
+};
+static StaticNeed static_need(int rows, int out_features, GemvPlan plan) {
+    const int n_groups = out_features / 128;
+    if (linear_small_uses_atomics(rows, n_groups, plan))
+        return {0, linear_small_counter_ints(rows, out_features) * sizeof(int32_t)};
+    return {(size_t)plan.n_partials() * rows * out_features * sizeof(float),
+            (size_t)n_groups * sizeof(int32_t)};
+}
+
+}  // namespace exl3
+
 EXL3_EXPORT size_t exl3_linear_static_need_bytes(int rows, int in_features, int out_features) {
     using namespace exl3;
     if (rows < 1 || rows > kLinearSmallMaxRows || in_features < 128 || out_features < 128) return 0;
-    const GemvPlan plan = plan_linear_small_launch(rows, in_features / 16, out_features / 128);
-    if (linear_small_uses_atomics(rows, out_features / 128, plan))
-        return linear_small_counter_ints(rows, out_features) * sizeof(int32_t);
-    return (size_t)plan.n_partials() * rows * out_features * sizeof(float);
+    // the launch plan depends on K (deeper splits from K = 5 on): the larger of the two
+    size_t need = 0;
+    for (int K : {4, 8}) {
+        const GemvPlan plan = plan_linear_small_launch(rows, in_features / 16, out_features / 128, K);
+        const size_t n = static_need(rows, out_features, plan).larger();
+        if (n > need) need = n;
+    }
+    return need;
 }
 
 EXL3_EXPORT int exl3_linear_forward_static(const uint16_t* x, int rows, const uint16_t* trellis,
@@ -250,8 +272,8 @@ EXL3_EXPORT int exl3_linear_forward_static(const uint16_t* x, int rows, const ui
     if (n_sub > 1 && (!group_sub || !suh)) return EXL3_E_BAD_INDEX;
     const int n_groups = out_tiles / 8;
     const GemvPlan plan = plan_linear_small_launch(rows, in_tiles, n_groups, K);
-    const size_t need = exl3_linear_static_need_bytes(rows, in_tiles * 16, out_tiles * 16);
-    if (need > kStaticPartialBytes || (size_t)n_groups * sizeof(int32_t) > kStaticCounterBytes)
+    const StaticNeed need = static_need(rows, out_tiles * 16, plan);
+    if (need.partial_bytes > kStaticPartialBytes || need.counter_bytes > kStaticCounterBytes)
         return EXL3_E_STATIC_LIMIT;
     hipStream_t s = as_stream(stream);
     unsigned char* base = nullptr;
