@@ -151,6 +151,45 @@ def test_accumulator_reduction_of_gate_up(cuda, oracle, tokens, top_k, E, D, H, 
         assert rel_l2(ya.cpu().numpy(), ref) <= TOL
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_random_shapes_three_reductions_agree(cuda, seed):
+    """Random small shapes (D and H from one to six Hadamard blocks, K from 2 to 8, both
+    codebooks, 1..40 tokens, top-k up to 6, few or many experts, indices outside the
+    expert range included: they are clamped): the two-launch chain with whatever kernels
+    the library picks (accumulators / grouped slots / per-slot partial rows), the same
+    with partial rows only, and the five-launch chain must agree to fp16 ulps."""
+    from ponyexl3_amd import EXL3SwitchGLU, ops
+
+    rng = np.random.default_rng(9000 + seed)
+    D, H = 128 * int(rng.integers(1, 7)), 128 * int(rng.integers(1, 7))
+    k = int(rng.integers(2, 9))
+    cb = int(rng.integers(0, 2))
+    E = int(rng.choice([2, 5, 16, 70]))
+    top_k = int(rng.integers(1, min(E, 6) + 1))
+    tokens = int(rng.choice([1, 2, 3, 7, 16, 40]))
+    act = int(rng.integers(0, 2))
+    rnd = lambda *s: torch.from_numpy(rng.integers(-32768, 32768, size=s, dtype=np.int16)).to(cuda)
+    sgn = lambda *s: torch.from_numpy(np.where(rng.random(s) > 0.5, -1.0, 1.0).astype(np.float16)).to(cuda)
+    gu, dn = rnd(D // 16, E * 2 * H // 16, 16 * k), rnd(H // 16, E * D // 16, 16 * k)
+    gu_suh, gu_svh, dn_suh, dn_svh = sgn(E, 2, D), sgn(E, 2 * H), sgn(E, H), sgn(E, D)
+    x = torch.from_numpy((rng.standard_normal((tokens, D)) * 0.25).astype(np.float16)).to(cuda)
+    idx = np.stack([rng.permutation(E)[:top_k] for _ in range(tokens)]).astype(np.int32)
+    if tokens > 1:
+        idx[0, 0], idx[-1, -1] = -3, E + 5  # clamped to expert 0 and E - 1
+    it = torch.from_numpy(idx).to(cuda)
+    args = (x, it, gu, gu_suh, gu_svh, dn, dn_suh, dn_svh, k, cb, act)
+    print(f"moe random seed={seed} D={D} H={H} k={k} cb={cb} E={E} top_k={top_k} tokens={tokens}", flush=True)
+    y = ops.moe_forward(*args)
+    y_rows = ops.moe_forward(*args, accumulators=False)
+    y_five = ops.moe_forward(*args, fused=False)
+    assert torch.equal(y, ops.moe_forward(*args))
+    assert int(ops.sync_counters(cuda, 1).abs().sum()) == 0
+    assert torch.isfinite(y.float()).all()
+    ref = y_five.float().cpu().numpy()
+    assert rel_l2(y.float().cpu().numpy(), ref) <= TOL
+    assert rel_l2(y_rows.float().cpu().numpy(), ref) <= TOL
+
+
 @pytest.mark.parametrize("tokens,act", [(40, "silu"), (200, "gelu")])
 def test_prefill_path_matches_oracle_and_slot_kernels(cuda, oracle, tokens, act):
     """From 24 tokens on the pairs are sorted by expert and go through the segmented
