@@ -267,6 +267,38 @@ def test_one_launch_layer_equals_three_launch_chain(cuda, rows, k, n_in, n_out):
     assert int(ops.sync_counters(cuda, 1).abs().sum()) == 0
 
 
+@pytest.mark.parametrize("seed", range(14))
+def test_random_shapes_all_paths_agree(cuda, oracle, seed):
+    """Random layers (1..40 Hadamard blocks in, 1..24 out, K = 1..8, three codebooks, with
+    and without bias) at random row counts up to 40: whatever kernel the library picks
+    with counters (accumulator or partial-row reduction, half-block or two-block splits,
+    eight-wave workgroups, medium-batch kernel, prefill GEMM) against the chained kernels
+    without counters and against the oracle; bit-identical call after call."""
+    from ponyexl3_amd import make_exl3_layer, ops
+
+    rng = np.random.default_rng(7000 + seed)
+    n_in, n_out = 128 * int(rng.integers(1, 41)), 128 * int(rng.integers(1, 25))
+    k, cb = int(rng.integers(1, 9)), int(rng.integers(0, 3))
+    rows = int(rng.choice([1, 1, 2, 3, 5, 8, 9, 16, 27, 40]))
+    has_bias = bool(rng.integers(0, 2))
+    layer = make_exl3_layer(k=k, in_features=n_in, out_features=n_out, seed=seed, mcg=cb == 1, mul1=cb == 2,
+                            bias=has_bias)
+    tr = ops.as_trellis_tensor(layer.trellis, cuda)
+    suh, svh = torch.from_numpy(layer.suh).to(cuda), torch.from_numpy(layer.svh).to(cuda)
+    bias = torch.from_numpy(layer.bias).to(cuda) if has_bias else None
+    xn = rng.standard_normal((rows, n_in)).astype(np.float16)
+    x = torch.from_numpy(xn).to(cuda)
+    print(f"linear random seed={seed} {n_in}x{n_out} k={k} cb={cb} rows={rows} bias={has_bias}", flush=True)
+    a = ops.linear_forward(x, tr, k, cb, suh, svh, bias, fused=True)
+    assert torch.equal(a, ops.linear_forward(x, tr, k, cb, suh, svh, bias, fused=True))
+    assert int(ops.sync_counters(cuda, 1).abs().sum()) == 0
+    b = ops.linear_forward(x, tr, k, cb, suh, svh, bias, fused=False)
+    want = oracle.linear_forward(layer.trellis, k, cb, layer.suh, layer.svh, xn,
+                                 bias=layer.bias if has_bias else None)
+    assert rel_l2(a.cpu().numpy(), want) <= 1e-3
+    assert rel_l2(b.cpu().numpy(), want) <= 1e-3
+
+
 @pytest.mark.parametrize("rows", [9, 13, 16, 17, 25, 32])
 @pytest.mark.parametrize("k,cb,n_in,n_out", [(4, 0, 2176, 640), (3, 1, 4096, 384), (5, 0, 1024, 1280),
                                              (8, 2, 1152, 256), (7, 0, 640, 128), (6, 1, 2048, 256),
