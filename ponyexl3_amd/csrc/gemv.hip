@@ -371,27 +371,23 @@ __global__ __launch_bounds__(NW * 64) void linear_small_kernel(
             const float* src = partial + (size_t)m * out_total + col;
             const size_t stride = (size_t)rows * out_total;
             float a = 0.f, b = 0.f;
-            int s = 0;
-            for (; s + 16 <= wg_splits; s += 16) {
+            // (a batch that runs past the last partial row re-reads that row and drops
+            // it: every batch is one round trip, whatever wg_splits is)
+            for (int s = 0; s < wg_splits; s += 16) {
                 uint64_t v[16];
 #pragma unroll
                 for (int i = 0; i < 16; i++)
                     v[i] = __hip_atomic_load(
-                        reinterpret_cast<const uint64_t*>(src + (size_t)(s + i) * stride),
+                        reinterpret_cast<const uint64_t*>(src + (size_t)min(s + i, wg_splits - 1) * stride),
                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
-                    const float2_t f = __builtin_bit_cast(float2_t, v[i]);
-                    a = __fadd_rn(a, f.x);
-                    b = __fadd_rn(b, f.y);
+                    if (s + i < wg_splits) {
+                        const float2_t f = __builtin_bit_cast(float2_t, v[i]);
+                        a = __fadd_rn(a, f.x);
+                        b = __fadd_rn(b, f.y);
+                    }
                 }
-            }
-            for (; s < wg_splits; s++) {
-                const float2_t f = __builtin_bit_cast(
-                    float2_t, __hip_atomic_load(reinterpret_cast<const uint64_t*>(src + (size_t)s * stride),
-                                                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-                a = __fadd_rn(a, f.x);
-                b = __fadd_rn(b, f.y);
             }
             a = (float)(half_t)a;
             b = (float)(half_t)b;

@@ -198,14 +198,25 @@ __device__ __forceinline__ bool moe_publish(float* row, float2_t v, int* counter
     return __shfl(seen, 0, kWave) == expected - 1;
 }
 
+// Eight partial rows in flight (a batch that runs past the last row re-reads that row and
+// drops it, so that every batch is one round trip); added in index order.
 __device__ __forceinline__ float2_t moe_sum_rows(const float* rows, int n, int lane) {
     float a = 0.f, b = 0.f;
-    for (int i = 0; i < n; i++) {
-        const float2_t f = __builtin_bit_cast(
-            float2_t, __hip_atomic_load(reinterpret_cast<const uint64_t*>(rows + i * 128 + 2 * lane),
-                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-        a = __fadd_rn(a, f.x);
-        b = __fadd_rn(b, f.y);
+    for (int s = 0; s < n; s += 8) {
+        uint64_t v[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+            v[i] = __hip_atomic_load(
+                reinterpret_cast<const uint64_t*>(rows + (size_t)min(s + i, n - 1) * 128 + 2 * lane),
+                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            if (s + i < n) {
+                const float2_t f = __builtin_bit_cast(float2_t, v[i]);
+                a = __fadd_rn(a, f.x);
+                b = __fadd_rn(b, f.y);
+            }
+        }
     }
     return float2_t{a, b};
 }
@@ -624,17 +635,27 @@ __global__ __launch_bounds__(NW * 64) void moe_gateup_grouped_kernel(
     const float* rows_g = part + (((size_t)sr * 2) * hblocks + hg) * n_wg * 128;
     const float* rows_u = part + (((size_t)sr * 2 + 1) * hblocks + hg) * n_wg * 128;
     float2_t sg{0.f, 0.f}, su{0.f, 0.f};
-    for (int i = 0; i < n_wg; i++) {
-        const float2_t fg = __builtin_bit_cast(
-            float2_t, __hip_atomic_load(reinterpret_cast<const uint64_t*>(rows_g + i * 128 + 2 * lane),
-                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-        const float2_t fu = __builtin_bit_cast(
-            float2_t, __hip_atomic_load(reinterpret_cast<const uint64_t*>(rows_u + i * 128 + 2 * lane),
-                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-        sg.x = __fadd_rn(sg.x, fg.x);
-        sg.y = __fadd_rn(sg.y, fg.y);
-        su.x = __fadd_rn(su.x, fu.x);
-        su.y = __fadd_rn(su.y, fu.y);
+    for (int s0 = 0; s0 < n_wg; s0 += 4) {  // four rows of each projection per round trip
+        uint64_t vg[4], vu[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const size_t off = (size_t)min(s0 + i, n_wg - 1) * 128 + 2 * lane;
+            vg[i] = __hip_atomic_load(reinterpret_cast<const uint64_t*>(rows_g + off),
+                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            vu[i] = __hip_atomic_load(reinterpret_cast<const uint64_t*>(rows_u + off),
+                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            if (s0 + i < n_wg) {
+                const float2_t fg = __builtin_bit_cast(float2_t, vg[i]);
+                const float2_t fu = __builtin_bit_cast(float2_t, vu[i]);
+                sg.x = __fadd_rn(sg.x, fg.x);
+                sg.y = __fadd_rn(sg.y, fg.y);
+                su.x = __fadd_rn(su.x, fu.x);
+                su.y = __fadd_rn(su.y, fu.y);
+            }
+        }
     }
     const half_t* svh_e = gu_svh + (size_t)e * 2 * H + hg * 128 + 2 * lane;
     float g0, g1, u0, u1;
