@@ -391,14 +391,18 @@ int linear_mid_max_rows() {
 
 // Splits of the reduction: enough workgroups for kWgPerCu per CU, but never more
 // than kMaxSplits partial rows per output (each costs a write and a read of
-// rows x out floats).
+// rows x out floats, and the finishing workgroup fetches eight of them per round
+// trip) - or twice that where a split then still has eight blocks to stream
+// (17408 -> 5120 at 16 rows: 8 splits = 320 workgroups 34.0 us, 16 splits 29.8 us;
+// with four or five blocks per split the extra splits cost more than they gain).
 MidPlan plan_linear_mid(int rows, int in_tiles, int n_groups) {
     (void)rows;
     static const int kWgPerCu = env_int("EXL3_LINEAR_MID_WG_PER_CU", 4, 1, 16);
     static const int kMaxSplits = env_int("EXL3_LINEAR_MID_MAX_SPLITS", 8, 1, 256);
     const int n_blocks = in_tiles / 8;
     int want = (256 * kWgPerCu + n_groups - 1) / (n_groups > 0 ? n_groups : 1);
-    if (want > kMaxSplits) want = kMaxSplits;
+    if (want >= 2 * kMaxSplits && n_blocks >= 2 * kMaxSplits * 8) want = 2 * kMaxSplits;
+    else if (want > kMaxSplits) want = kMaxSplits;
     if (want > n_blocks) want = n_blocks;
     if (want < 1) want = 1;
     const int blocks_per_split = (n_blocks + want - 1) / want;
