@@ -461,7 +461,7 @@ def bench_ceilings(dev):
 
     from ponyexl3_amd import _lib
 
-    lib = _lib.load()
+    lib = _lib.load_diag()
     total = 2 << 30
     buf = torch.randint(-2**31, 2**31 - 1, (total // 4,), dtype=torch.int32, device=dev)
     out = torch.zeros(4096 * 1024, dtype=torch.float32, device=dev)

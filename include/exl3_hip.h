@@ -40,38 +40,13 @@ extern "C" {
 #define EXL3_E_BAD_INDEX (-7)     /* tile_sub / expert index table inconsistent */
 #define EXL3_E_UNSUPPORTED (-8)   /* valid request this build has no kernel for */
 #define EXL3_E_STATIC_LIMIT (-9)  /* exl3_linear_forward_static: beyond its built-in scratch */
+#define EXL3_E_INCOMPLETE (-10)   /* exl3_counters_status: a split reduction gave up waiting */
 
 /* Library version (major*10000 + minor*100 + patch). */
 int exl3_version(void);
 
 /* Human-readable text for a status code; never NULL. */
 const char *exl3_status_string(int status);
-
-/*
- * Diagnostics for measured ceilings (no counterpart in the reference; its kernel
- * benches quote Gw/s only, tools/bench/gemv_split_bench.py:51,84).
- * exl3_diag_stream_read: reads `bytes` (16-byte aligned buffer) once with streaming
- *   loads; out: 4 bytes of device memory, practically never written.
- * exl3_diag_decode_loop: n_wg workgroups of 16 waves run `steps` (a multiple of 4)
- *   iterations of the small-batch kernels' inner loop (one wave-wide load of 256*K
- *   bytes, per-lane decode of 32 codewords, 8 matrix-pipe dot products) over
- *   consecutive 256*K-byte rows of buf, wrapping at the largest power-of-two row
- *   count that fits in `bytes`; weights per launch = n_wg*16*steps*2048. cb 0 or 1.
- *   out: float [n_wg*1024].
- * exl3_diag_empty_launch: a kernel that does nothing on a grid of grid_x * grid_y
- *   workgroups of `threads` lanes (a multiple of 64, at most 1024): what the dispatch of
- *   such a grid costs.
- * exl3_diag_first_rows: on the same kind of grid every wave requests its first four
- *   tile rows (wave-wide loads of 256*K bytes, rows row_base + 4*wave .. +3 of buf,
- *   wrapping like above), waits for them and leaves: the time before a small-batch
- *   launch can decode anything. out: 4 bytes of device memory, practically never written.
- */
-int exl3_diag_stream_read(const void *buf, size_t bytes, void *out, void *stream);
-int exl3_diag_decode_loop(const void *buf, size_t bytes, int K, int cb, int n_wg, int steps,
-                          float *out, void *stream);
-int exl3_diag_empty_launch(int grid_x, int grid_y, int threads, void *stream);
-int exl3_diag_first_rows(const void *buf, size_t bytes, int K, int grid_x, int grid_y,
-                         int threads, unsigned row_base, void *out, void *stream);
 
 /* Largest row count the small-batch kernel (exl3_gemv) accepts per call. */
 int exl3_gemv_max_rows(void);
@@ -277,6 +252,9 @@ size_t exl3_gemm_workspace_bytes(int rows, int in_tiles, int tn_count);
  *            rotation, then everything else). NULL selects the three-launch chain
  *            (exl3_had128_pre, exl3_gemv_partials, exl3_had128_post) resp. the
  *            prefill GEMM.
+ *            Status word: when counters_len is at least two ints more than the call
+ *            needs, the LAST int of the array is a sticky status word (see
+ *            exl3_counters_status below).
  */
 int exl3_linear_forward(const uint16_t *x, int rows, const uint16_t *trellis, int in_tiles,
                         int out_tiles, int K, int cb, const uint16_t *suh, int n_sub,
@@ -285,6 +263,25 @@ int exl3_linear_forward(const uint16_t *x, int rows, const uint16_t *trellis, in
                         size_t counters_len, void *stream);
 
 size_t exl3_linear_workspace_bytes(int rows, int in_features, int out_features, int n_sub);
+
+/*
+ * Error channel of the accumulator reductions (exl3_linear_forward, exl3_moe_forward,
+ * exl3_linear_forward_static); no counterpart in the reference, whose kernels have no
+ * split state that outlives a launch. The workgroup that finishes a 128-column group
+ * may have to wait for atomic adds of other workgroups that are already in flight; that
+ * wait is bounded (EXL3_SPIN_LIMIT polls, default 2^22). It can only run out when the
+ * contract of the counters array was broken (not all zero on entry, or shared by calls
+ * that overlap). Then no total can be trusted: the workgroup writes NaN to the outputs
+ * of its group (for the MoE chain: to that block of the down projection's input, hence
+ * to the slot's output), sets the status word - the last int of the counters array as
+ * passed to the call, provided the array is at least two ints longer than the call
+ * needs - to a non-zero value and leaves the accumulators as they are. The caller
+ * must zero the whole array before using it again.
+ * exl3_counters_status waits for `stream`, reads that word (counters_len as passed to
+ * the forward call; counters == NULL: the array of exl3_linear_forward_static on the
+ * current device) and returns EXL3_OK or EXL3_E_INCOMPLETE.
+ */
+int exl3_counters_status(const int32_t *counters, size_t counters_len, void *stream);
 
 /*
  * exl3_linear_forward for callers that cannot allocate device memory or carry a
@@ -304,7 +301,10 @@ size_t exl3_linear_workspace_bytes(int rows, int in_features, int out_features, 
  *   launched).
  * All calls on one GPU share that GPU's array: calls that overlap there (two
  * streams, two threads) race. The counter half is all zero whenever no call is
- * running.
+ * running. The first call on a device clears the counter half on `stream` and waits
+ * for that to complete before it launches anything else; it must not be made while
+ * `stream` is being captured into a graph (EXL3_E_UNSUPPORTED, nothing is launched):
+ * call once eagerly before capturing.
  */
 size_t exl3_linear_static_scratch_bytes(void);
 size_t exl3_linear_static_need_bytes(int rows, int in_features, int out_features);
@@ -340,6 +340,8 @@ int exl3_linear_forward_static(const uint16_t *x, int rows, const uint16_t *trel
  *               its own and the launch issues at most EXL3_MOE_MAX_ATOMICS = 300000
  *               atomics); the result can differ from the partial-row reduction by
  *               an fp16 ulp, and is bit-identical from call to call either way.
+ *               Two more ints than that make the last int the status word of
+ *               exl3_counters_status.
  * Only the selected experts' trellis blocks are read. In the two-launch chain, with
  * 2 <= tokens, at most 512 slots and at least one slot per two experts, the slots that
  * route to one expert share a pass over its weights (four batch rows per pass; same

@@ -12,6 +12,7 @@ import os
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libexl3_hip.so")
+DIAG_LIB_PATH = os.path.join(_PKG_DIR, "libexl3_diag.so")
 
 EXL3_OK = 0
 EXL3_E_BAD_K = -1
@@ -23,6 +24,7 @@ EXL3_E_LAUNCH = -6
 EXL3_E_BAD_INDEX = -7
 EXL3_E_UNSUPPORTED = -8
 EXL3_E_STATIC_LIMIT = -9
+EXL3_E_INCOMPLETE = -10
 
 _vp = ctypes.c_void_p
 _i = ctypes.c_int
@@ -32,10 +34,6 @@ _sz = ctypes.c_size_t
 PROTOTYPES = {
     "exl3_version": (_i, []),
     "exl3_status_string": (ctypes.c_char_p, [_i]),
-    "exl3_diag_stream_read": (_i, [_vp, _sz, _vp, _vp]),
-    "exl3_diag_decode_loop": (_i, [_vp, _sz, _i, _i, _i, _i, _vp, _vp]),
-    "exl3_diag_empty_launch": (_i, [_i, _i, _i, _vp]),
-    "exl3_diag_first_rows": (_i, [_vp, _sz, _i, _i, _i, _i, ctypes.c_uint, _vp, _vp]),
     "exl3_gemv_max_rows": (_i, []),
     "exl3_linear_small_max_rows": (_i, []),
     "exl3_decode_full": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _vp]),
@@ -65,6 +63,7 @@ PROTOTYPES = {
         [_vp, _i, _vp, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _sz, _vp],
     ),
     "exl3_linear_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "exl3_counters_status": (_i, [_vp, _sz, _vp]),
     "exl3_linear_static_scratch_bytes": (_sz, []),
     "exl3_linear_static_need_bytes": (_sz, [_i, _i, _i]),
     "exl3_linear_forward_static": (
@@ -78,7 +77,16 @@ PROTOTYPES = {
     "exl3_moe_workspace_bytes": (_sz, [_i, _i, _i, _i]),
 }
 
+# libexl3_diag.so (include/exl3_diag.h): measurement probes, not part of the product library
+DIAG_PROTOTYPES = {
+    "exl3_diag_stream_read": (_i, [_vp, _sz, _vp, _vp]),
+    "exl3_diag_decode_loop": (_i, [_vp, _sz, _i, _i, _i, _i, _vp, _vp]),
+    "exl3_diag_empty_launch": (_i, [_i, _i, _i, _vp]),
+    "exl3_diag_first_rows": (_i, [_vp, _sz, _i, _i, _i, _i, ctypes.c_uint, _vp, _vp]),
+}
+
 _lib = None
+_diag = None
 
 
 def load() -> ctypes.CDLL:
@@ -101,6 +109,23 @@ def load() -> ctypes.CDLL:
     return _lib
 
 
+def load_diag() -> ctypes.CDLL:
+    """Load libexl3_diag.so, the measurement probes bench.py reports its ceilings from."""
+    global _diag
+    if _diag is None:
+        if not os.path.exists(DIAG_LIB_PATH):
+            raise RuntimeError(f"{DIAG_LIB_PATH} is missing: run `python -m ponyexl3_amd.build`")
+        import torch  # noqa: F401
+
+        lib = ctypes.CDLL(DIAG_LIB_PATH)
+        for name, (restype, argtypes) in DIAG_PROTOTYPES.items():
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _diag = lib
+    return _diag
+
+
 def status_string(status: int) -> str:
     return load().exl3_status_string(int(status)).decode()
 
@@ -111,6 +136,6 @@ def check(status: int, what: str) -> None:
     if status == EXL3_OK:
         return
     msg = f"{what}: {status_string(status)} (status {status})"
-    if status == EXL3_E_LAUNCH:
+    if status in (EXL3_E_LAUNCH, EXL3_E_INCOMPLETE):
         raise RuntimeError(msg)
     raise ValueError(msg)

@@ -3,7 +3,8 @@
 ``python -m ponyexl3_amd.build`` or ``ponyexl3_amd.build.build()``. Each .hip
 file is one translation unit compiled in parallel; the objects are linked into
 ``ponyexl3_amd/libexl3_hip.so``, the C-ABI library declared in
-``include/exl3_hip.h``.
+``include/exl3_hip.h``, and (``diag.hip`` alone) ``ponyexl3_amd/libexl3_diag.so``,
+the measurement probes declared in ``include/exl3_diag.h``.
 """
 
 from __future__ import annotations
@@ -19,7 +20,10 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(PKG_DIR, "libexl3_hip.so")
 
-SOURCES = ["decode.hip", "hadamard.hip", "gemv.hip", "linear_mid.hip", "gemm.hip", "moe.hip", "search.hip", "diag.hip", "capi.hip"]
+SOURCES = ["decode.hip", "hadamard.hip", "gemv.hip", "linear_mid.hip", "gemm.hip", "moe.hip", "search.hip", "capi.hip"]
+# measurement probes (include/exl3_diag.h): a library of their own, kept out of the product ABI
+DIAG_SOURCES = ["diag.hip"]
+DIAG_LIB_PATH = os.path.join(PKG_DIR, "libexl3_diag.so")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -57,15 +61,17 @@ def _compile(src: str, extra: list[str]) -> str:
 def build(verbose: bool = False, jobs: int | None = None, extra_flags: list[str] | None = None) -> str:
     os.makedirs(OBJ_DIR, exist_ok=True)
     extra = list(extra_flags or [])
-    jobs = jobs or min(len(SOURCES), int(os.environ.get("MAX_JOBS", "8")))
+    every = SOURCES + DIAG_SOURCES
+    jobs = jobs or min(len(every), int(os.environ.get("MAX_JOBS", "8")))
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
-        objs = list(pool.map(lambda s: _compile(s, extra), SOURCES))
-    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]
-    proc = subprocess.run(cmd, capture_output=True, text=True)
-    if proc.returncode != 0:
-        raise RuntimeError(f"link failed:\n{proc.stderr[-4000:]}")
-    if verbose:
-        print(f"built {LIB_PATH} ({os.path.getsize(LIB_PATH)} bytes)")
+        objs = list(pool.map(lambda s: _compile(s, extra), every))
+    for path, group in ((LIB_PATH, objs[: len(SOURCES)]), (DIAG_LIB_PATH, objs[len(SOURCES):])):
+        cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", path, *group]
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"link failed:\n{proc.stderr[-4000:]}")
+        if verbose:
+            print(f"built {path} ({os.path.getsize(path)} bytes)")
     return LIB_PATH
 
 

@@ -58,6 +58,9 @@ EXL3_EXPORT const char* exl3_status_string(int status) {
         case EXL3_E_UNSUPPORTED: return "no kernel for this request";
         case EXL3_E_STATIC_LIMIT:
             return "request needs more scratch than the built-in array of exl3_linear_forward_static holds";
+        case EXL3_E_INCOMPLETE:
+            return "a split reduction gave up waiting (counters not zero on entry, or shared by "
+                   "overlapping calls); the affected outputs are NaN and the counters must be zeroed";
         default: return "unknown status";
     }
 }
@@ -94,10 +97,12 @@ EXL3_EXPORT int exl3_linear_forward(const uint16_t* x, int rows, const uint16_t*
         if (counters) {
             // one launch: rotation, GEMV, split reduction and output transform fused;
             // the counters array holds the 64-bit accumulators (two ints each)
-            if (counters_len < linear_small_counter_ints(rows, out_features)) return EXL3_E_WORKSPACE;
+            const size_t need = linear_small_counter_ints(rows, out_features);
+            if (counters_len < need) return EXL3_E_WORKSPACE;
             return launch_linear_small(x, rows, trellis, in_tiles, out_tiles, K, cb, suh, n_sub,
                                        group_sub, svh, bias, y, partial, counters,
-                                       plan_linear_small_launch(rows, in_tiles, n_groups, K), s);
+                                       plan_linear_small_launch(rows, in_tiles, n_groups, K), s,
+                                       counters_status_word(counters, counters_len, need));
         }
         if (int rc = launch_had_pre(x, rows, in_features, suh, n_sub, xh, s)) return rc;
         if (int rc = launch_gemv_partials(xh, rows, n_sub, trellis, in_tiles, out_tiles, K, cb,
@@ -200,27 +205,45 @@ static __device__ __align__(256) unsigned char scratch[exl3::kStaticScratchBytes
 
 namespace exl3 {
 
-// Device address of this GPU's copy of `scratch` (resolved on first use, with that
-// device current); the array is cleared once by a fill kernel on `stream` (every
-// launch leaves the accumulators it used at zero).
+// Device address of this GPU's copy of `scratch`, resolved on first use with that
+// device current. The counter half is cleared once by a fill kernel on `stream`, and the
+// address is published only after that fill has completed (a stream synchronisation:
+// it allocates nothing), so a later first call on another stream cannot overtake it.
+// The first use on a device must not happen under stream capture (the fill and the
+// synchronisation cannot be captured): such a call is refused with EXL3_E_UNSUPPORTED
+// and nothing is launched; one eager call beforehand is enough.
+static unsigned char* g_static_ptrs[kStaticMaxDevices];  // zero-initialised; one slot per device
+static std::mutex g_static_lock;
+
 static int static_scratch(hipStream_t stream, unsigned char** out) {
-    static unsigned char* ptrs[kStaticMaxDevices];  // zero-initialised; one slot per device
-    static std::mutex lock;
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kStaticMaxDevices)
         return EXL3_E_LAUNCH;
-    std::lock_guard<std::mutex> guard(lock);
-    if (!ptrs[dev]) {
+    std::lock_guard<std::mutex> guard(g_static_lock);
+    if (!g_static_ptrs[dev]) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &capturing) != hipSuccess ||
+            capturing != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            return EXL3_E_UNSUPPORTED;
+        }
         void* p = nullptr;
         if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return EXL3_E_LAUNCH;
         const int n_ints = (int)(kStaticCounterBytes / sizeof(int32_t));
         static_zero_kernel<<<dim3((unsigned)((n_ints + 255) / 256)), dim3(256), 0, stream>>>(
             reinterpret_cast<int32_t*>(static_cast<unsigned char*>(p) + kStaticPartialBytes), n_ints);
         if (int rc = launch_status()) return rc;
-        ptrs[dev] = static_cast<unsigned char*>(p);
+        if (hipStreamSynchronize(stream) != hipSuccess) return EXL3_E_LAUNCH;
+        g_static_ptrs[dev] = static_cast<unsigned char*>(p);
     }
-    *out = ptrs[dev];
+    *out = g_static_ptrs[dev];
     return EXL3_OK;
+}
+
+// Status word of the static array: the last int of the counter half (static_need keeps
+// the accumulators out of the last eight bytes).
+static int* static_status_word(unsigned char* base) {
+    return reinterpret_cast<int*>(base + kStaticScratchBytes) - 1;
 }
 
 }  // namespace exl3
@@ -273,12 +296,37 @@ EXL3_EXPORT int exl3_linear_forward_static(const uint16_t* x, int rows, const ui
     const int n_groups = out_tiles / 8;
     const GemvPlan plan = plan_linear_small_launch(rows, in_tiles, n_groups, K);
     const StaticNeed need = static_need(rows, out_tiles * 16, plan);
-    if (need.partial_bytes > kStaticPartialBytes || need.counter_bytes > kStaticCounterBytes)
+    if (need.partial_bytes > kStaticPartialBytes || need.counter_bytes > kStaticCounterBytes - 8)
         return EXL3_E_STATIC_LIMIT;
     hipStream_t s = as_stream(stream);
     unsigned char* base = nullptr;
     if (int rc = static_scratch(s, &base)) return rc;
     return launch_linear_small(x, rows, trellis, in_tiles, out_tiles, K, cb, suh, n_sub, group_sub,
                                svh, bias, y, reinterpret_cast<float*>(base),
-                               reinterpret_cast<int*>(base + kStaticPartialBytes), plan, s);
+                               reinterpret_cast<int*>(base + kStaticPartialBytes), plan, s,
+                               static_status_word(base));
+}
+
+// Whether a finishing workgroup of an accumulator reduction gave up on this counters
+// array since it was last zeroed. Waits for `stream`, then reads the status word.
+EXL3_EXPORT int exl3_counters_status(const int32_t* counters, size_t counters_len, void* stream) {
+    using namespace exl3;
+    hipStream_t s = as_stream(stream);
+    const int* word = nullptr;
+    if (counters) {
+        if (counters_len < 2) return EXL3_E_BAD_SHAPE;
+        word = counters + (counters_len - 1);
+    } else {
+        int dev = -1;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kStaticMaxDevices)
+            return EXL3_E_LAUNCH;
+        std::lock_guard<std::mutex> guard(g_static_lock);
+        if (!g_static_ptrs[dev]) return EXL3_OK;  // never used on this device
+        word = static_status_word(g_static_ptrs[dev]);
+    }
+    int host = 0;
+    if (hipMemcpyAsync(&host, word, sizeof(int), hipMemcpyDeviceToHost, s) != hipSuccess ||
+        hipStreamSynchronize(s) != hipSuccess)
+        return EXL3_E_LAUNCH;
+    return host ? EXL3_E_INCOMPLETE : EXL3_OK;
 }

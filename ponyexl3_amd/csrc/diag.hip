@@ -4,6 +4,7 @@
 // Hadamard, no split reduction, no launch-bound phases). They compute nothing a
 // caller needs; they exist so that roofline fractions can be quoted against
 // measured as well as published peaks.
+#include "../../include/exl3_diag.h"
 #include "exl3_device.hpp"
 #include "exl3_host.hpp"
 #include "exl3_small.hpp"

@@ -88,7 +88,9 @@ int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, in
                         int out_tiles, int K, int cb, const uint16_t* suh, int n_sub,
                         const int32_t* group_sub, const uint16_t* svh, const uint16_t* bias,
                         uint16_t* y, float* partial, int* counters, GemvPlan plan,
-                        hipStream_t stream);
+                        hipStream_t stream, int* status = nullptr);
+// `status` (device, may be NULL): set to non-zero by a finishing workgroup of the
+// accumulator reduction whose bounded wait for the other contributors ran out.
 
 // Medium-batch layer (rows <= kLinearMidMaxRows) on rotated activations xh, fp16
 // [rows][n_sub][in]: weights decoded once and fed to 16x16x16 MFMA from registers;
@@ -167,6 +169,16 @@ inline int env_int(const char* name, int dflt, int lo, int hi) {
     if (!v || !*v) return dflt;
     const int x = atoi(v);
     return x < lo ? lo : (x > hi ? hi : x);
+}
+
+// Polls a finishing workgroup spends on accumulators whose counts are not complete yet
+// before it gives up (EXL3_SPIN_LIMIT; read at every launch so that a test can lower it).
+inline int reduction_spin_limit() { return env_int("EXL3_SPIN_LIMIT", 1 << 22, 1, 1 << 30); }
+
+// Where the status word of a counters array lives: its last int, if the array is at
+// least two ints longer than the launch needs (so that no accumulator shares it).
+inline int* counters_status_word(int32_t* counters, size_t counters_len, size_t needed) {
+    return counters && counters_len >= needed + 2 ? counters + (counters_len - 1) : nullptr;
 }
 
 }  // namespace exl3

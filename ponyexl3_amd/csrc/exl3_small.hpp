@@ -5,30 +5,11 @@
 #pragma once
 
 #include "exl3_device.hpp"
+#include "exl3_fixpoint.hpp"
 
 namespace exl3 {
 
 constexpr float kHadScaleF = 0.088388347648318440550f;  // 1/sqrt(128)
-
-// Accumulator word of the atomic split reductions: count << 56 | sum, the sum a signed
-// fixed-point number with 24 fraction bits (|partial sum| clamped to 2^18; fp16 ends at
-// 65504). Up to 255 contributors.
-constexpr float kFixScale = 16777216.f;  // 2^24
-constexpr float kFixClamp = 262144.f;    // 2^18
-
-__device__ __forceinline__ unsigned long long fix_word(float v) {
-    v = fminf(fmaxf(v, -kFixClamp), kFixClamp);
-    const long long fixed = (long long)((double)v * (double)kFixScale);
-    return (1ull << 56) + (unsigned long long)fixed;
-}
-__device__ __forceinline__ int fix_count(unsigned long long w) {
-    return (int)((long long)(w + (1ull << 55)) >> 56);
-}
-__device__ __forceinline__ float fix_value(unsigned long long w) {
-    const long long c = (long long)(w + (1ull << 55)) >> 56;
-    const long long fixed = (long long)(w - ((unsigned long long)c << 56));
-    return (float)((double)fixed * (1.0 / (double)kFixScale));
-}
 
 // Row stride (halfs) of a wave's staged activation block [MT][kXwLd]: 128 values
 // plus 16 bytes, so that the four batch rows a quad of lanes reads with one

@@ -195,7 +195,7 @@ __global__ __launch_bounds__(NW * 64) void linear_small_kernel(
     const half_t* __restrict__ suh, const half_t* __restrict__ svh,
     const half_t* __restrict__ bias, half_t* __restrict__ y, float* partial, int* counters,
     const int* __restrict__ group_sub, int in_tiles, int out_tiles, int rows, int n_groups,
-    int tk_per_split, int n_splits) {
+    int tk_per_split, int n_splits, int* status, int spin_limit) {
     static_assert(NW == 4 || (NW == 8 && ATOMIC), "eight-wave workgroups use the accumulators");
     __shared__ __attribute__((aligned(16))) half_t xs[NW][MT][kXwLd];
     const int g = blockIdx.x;
@@ -284,7 +284,8 @@ __global__ __launch_bounds__(NW * 64) void linear_small_kernel(
                 if (m < rows) ok = ok && fix_count(w0[m]) == wg_splits && fix_count(w1[m]) == wg_splits;
             return __ballot(ok) == ~0ull;
         };
-        for (int spin = 0; !all_complete() && spin < (1 << 22); spin++) {
+        bool complete = all_complete();
+        for (int spin = 0; !complete && spin < spin_limit; spin++) {
 #pragma unroll
             for (int m = 0; m < MT; m++) {
                 if (m < rows) {
@@ -293,6 +294,21 @@ __global__ __launch_bounds__(NW * 64) void linear_small_kernel(
                     w1[m] = __hip_atomic_load(slot + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
+            complete = all_complete();
+        }
+        if (!complete) {
+            // The counts never became complete (the array was not zero on entry, or it is
+            // shared with an overlapping call). No total can be trusted: the group's
+            // outputs become NaN, the status word is set and the accumulators are left
+            // as they are - the caller has to zero the array again.
+            if (status && lane == 0)
+                __hip_atomic_fetch_or(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            half2_t bad;
+            bad.x = bad.y = bits_to_half(0x7E00);
+#pragma unroll
+            for (int m = 0; m < MT; m++)
+                if (m < rows) *reinterpret_cast<half2_t*>(y + (size_t)m * out_total + col) = bad;
+            return;
         }
         half2_t sv, bv;
         if (svh) sv = *reinterpret_cast<const half2_t*>(svh + col);
@@ -533,9 +549,10 @@ int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, in
                         int out_tiles, int K, int cb, const uint16_t* suh, int n_sub,
                         const int32_t* group_sub, const uint16_t* svh, const uint16_t* bias,
                         uint16_t* y, float* partial, int* counters, GemvPlan plan,
-                        hipStream_t stream) {
+                        hipStream_t stream, int* status) {
     if (int rc = check_k_cb(K, cb)) return rc;
     if (!x || !trellis || !y || !counters) return EXL3_E_NULL_POINTER;
+    const int spin_limit = reduction_spin_limit();
     const bool atomic = linear_small_uses_atomics(rows, out_tiles / 8, plan);
     if (atomic && (reinterpret_cast<uintptr_t>(counters) & 7)) return EXL3_E_BAD_SHAPE;
     if (!atomic && !partial) return EXL3_E_NULL_POINTER;
@@ -562,7 +579,8 @@ int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, in
                         reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(suh),
                         reinterpret_cast<const half_t*>(svh), reinterpret_cast<const half_t*>(bias),
                         reinterpret_cast<half_t*>(y), partial, counters, group_sub, in_tiles,
-                        out_tiles, rows, n_groups, plan.tk_per_split, plan.n_splits);
+                        out_tiles, rows, n_groups, plan.tk_per_split, plan.n_splits, status,
+                        spin_limit);
             };
             if (atomic) launch(std::true_type{});
             else launch(std::false_type{});
@@ -574,7 +592,7 @@ int launch_linear_small(const uint16_t* x, int rows, const uint16_t* trellis, in
                     reinterpret_cast<const half_t*>(suh), reinterpret_cast<const half_t*>(svh),
                     reinterpret_cast<const half_t*>(bias), reinterpret_cast<half_t*>(y), partial,
                     counters, group_sub, in_tiles, out_tiles, rows, n_groups, plan.tk_per_split,
-                    plan.n_splits);
+                    plan.n_splits, status, spin_limit);
             return launch_status();
         }
         using T = std::true_type;

@@ -321,7 +321,8 @@ __global__ __launch_bounds__(512) void moe_gateup_pair_kernel(
     const uint32_t* __restrict__ gu_trellis, const half_t* __restrict__ x,
     const int* __restrict__ indices, const half_t* __restrict__ gu_suh,
     const half_t* __restrict__ gu_svh, const half_t* __restrict__ dn_suh, half_t* xh_dn,
-    unsigned long long* sums, int top_k, int E, int D, int H, int activation) {
+    unsigned long long* sums, int top_k, int E, int D, int H, int activation, int* status,
+    int spin_limit) {
     __shared__ __attribute__((aligned(16))) half_t xs[8][1][kXwLd];
     __shared__ float red[8][128];
     const int lane = threadIdx.x & 63;
@@ -369,10 +370,23 @@ __global__ __launch_bounds__(512) void moe_gateup_pair_kernel(
         for (int q = 0; q < 4; q++) ok = ok && fix_count(w[q]) == n_chunks;
         return __ballot(ok) == ~0ull;
     };
-    for (int spin = 0; !all_complete() && spin < (1 << 22); spin++) {
+    bool complete = all_complete();
+    for (int spin = 0; !complete && spin < spin_limit; spin++) {
 #pragma unroll
         for (int q = 0; q < 4; q++)
             w[q] = __hip_atomic_load(slot[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        complete = all_complete();
+    }
+    if (!complete) {
+        // the counts never became complete (array not zero on entry, or shared with an
+        // overlapping call): NaN for this block of the down projection's input (and so
+        // for the slot's output), status word set, accumulators left for the caller to zero
+        if (status && lane == 0)
+            __hip_atomic_fetch_or(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        half2_t bad;
+        bad.x = bad.y = bits_to_half(0x7E00);
+        *reinterpret_cast<half2_t*>(xh_dn + (size_t)s * H + hg * 128 + 2 * lane) = bad;
+        return;
     }
 #pragma unroll
     for (int q = 0; q < 4; q++)
@@ -1003,7 +1017,10 @@ EXL3_EXPORT int exl3_moe_forward(const uint16_t* x, int tokens, const int32_t* i
                         reinterpret_cast<const half_t*>(gu_svh),
                         reinterpret_cast<const half_t*>(dn_suh), xh_dn,
                         reinterpret_cast<unsigned long long*>(counters), top_k, num_experts, D, H,
-                        activation);
+                        activation,
+                        counters_status_word(counters, counters_len,
+                                             pair_ints + (size_t)slots * dblocks),
+                        reduction_spin_limit());
                 if (int rc = launch_status()) return rc;
                 moe_down_kernel<k.value, c.value, NW>
                     <<<dim3((unsigned)(slots * dblocks), (unsigned)((hblocks + 3) / 4)),

@@ -80,26 +80,36 @@ class FusedEXL3Group(torch.nn.Module):
         outs = torch.split(y, self._out_features, dim=-1)
         return tuple(o.reshape(lead + (n,)) for o, n in zip(outs, self._out_features))
 
-    def _same_input(self, x: torch.Tensor) -> bool:
+    def _same_input(self, x: torch.Tensor, idx: int | None = None) -> bool:
         """Whether x is the input the cached outputs were computed from. The reference
         compares object identity (ponyexl3/mlx/exl3_fused.py:204-208), which is enough
         for immutable mlx arrays. A torch tensor can be refilled in place (static
         decode buffers, HIP-graph inputs), so the version counter must match too; the
         tensor is held weakly (a freed tensor's address can be handed out again); and a
         result computed eagerly must not stand in for a launch that a graph capture
-        has to record."""
+        has to record. Tensors made under ``torch.inference_mode()`` keep no version
+        counter; for those a request is served from the cache only while it asks for a
+        member that has not been served from it yet (a second request for the same
+        member is a new step, whatever the tensor object is)."""
         if self._cache_out is None or self._cache_key is None:
             return False
         ref, version, capturing = self._cache_key
-        return (ref() is x and version == x._version
-                and capturing == (x.is_cuda and torch.cuda.is_current_stream_capturing()))
+        if ref() is not x or version != self._version_of(x):
+            return False
+        if version is None and (idx is None or idx in self._cache_served):
+            return False
+        return capturing == (x.is_cuda and torch.cuda.is_current_stream_capturing())
+
+    @staticmethod
+    def _version_of(x: torch.Tensor):
+        return None if x.is_inference() else x._version
 
     def cached(self, x: torch.Tensor, idx: int | None = None) -> tuple[torch.Tensor, ...]:
         """Outputs of all members for x, computed once per distinct input and dropped
         as soon as every member has been served (nothing is kept alive after that)."""
-        if not self._same_input(x):
+        if not self._same_input(x, idx):
             self._cache_out = self.forward_all(x)
-            self._cache_key = (weakref.ref(x), x._version,
+            self._cache_key = (weakref.ref(x), self._version_of(x),
                                x.is_cuda and torch.cuda.is_current_stream_capturing())
             self._cache_served = set()
         outs = self._cache_out

@@ -46,12 +46,19 @@ class _Shard:
 
     def __init__(self, path: str):
         self.path = path
+        size = os.path.getsize(path)
         with open(path, "rb") as f:
-            (hlen,) = struct.unpack("<Q", f.read(8))
+            head = f.read(8)
+            if len(head) < 8:
+                raise ValueError(f"{path}: too short for a safetensors file")
+            (hlen,) = struct.unpack("<Q", head)
+            if 8 + hlen > size:
+                raise ValueError(f"{path}: header of {hlen} bytes runs past the end of the file ({size} bytes)")
             header = json.loads(f.read(hlen))
         header.pop("__metadata__", None)
         self.entries: dict[str, dict] = header
         self._base = 8 + hlen
+        self._data_bytes = size - self._base
         self._map: mmap.mmap | None = None
 
     def names(self) -> Iterator[str]:
@@ -65,7 +72,10 @@ class _Shard:
         if self._map is None:
             with open(self.path, "rb") as f:
                 self._map = mmap.mmap(f.fileno(), 0, access=mmap.ACCESS_READ)
-        lo, hi = e["data_offsets"]
+        lo, hi = (int(v) for v in e["data_offsets"])
+        if not 0 <= lo <= hi <= self._data_bytes:
+            raise ValueError(f"{self.path}: tensor {name!r} has data offsets [{lo}, {hi}) outside the "
+                             f"{self._data_bytes} data bytes of the file")
         n = int(np.prod(e["shape"], dtype=np.int64)) if e["shape"] else 1
         if hi - lo != n * np.dtype(dt).itemsize:
             raise ValueError(f"{self.path}: tensor {name!r} has {hi - lo} bytes for shape {e['shape']}")
@@ -123,14 +133,23 @@ class Checkpoint:
             path = os.path.join(model_dir, rel)
             if os.path.isfile(path):
                 self._where[name] = path
+        self._scanned = False
         if len(self._where) < len(listed) or not listed:
             # no index, or one that names files that are not there: read the headers
-            for root, _dirs, files in sorted(os.walk(model_dir)):
-                for fn in sorted(files):
-                    if fn.endswith(".safetensors"):
-                        shard = self._shard(os.path.join(root, fn))
-                        for name in shard.names():
-                            self._where.setdefault(name, shard.path)
+            self._scan_shards()
+
+    def _scan_shards(self) -> None:
+        """Reads the header of every *.safetensors file below the directory once and
+        adds the tensors no index entry covers."""
+        if self._scanned:
+            return
+        self._scanned = True
+        for root, _dirs, files in sorted(os.walk(self.model_dir)):
+            for fn in sorted(files):
+                if fn.endswith(".safetensors"):
+                    shard = self._shard(os.path.join(root, fn))
+                    for name in shard.names():
+                        self._where.setdefault(name, shard.path)
 
     def _shard(self, path: str) -> _Shard:
         if path not in self._shards:
@@ -139,6 +158,17 @@ class Checkpoint:
 
     def has(self, tensor_name: str) -> bool:
         path = self._where.get(tensor_name)
+        if path is None or tensor_name not in self._shard(path).entries:
+            # an index may omit tensors that a shard holds (the reference looks through
+            # the shards per tensor, ponyexl3/ref/loader.py:108-125): scan once, then trust
+            # the table
+            self._scan_shards()
+            path = self._where.get(tensor_name)
+            if path is not None and tensor_name not in self._shard(path).entries:
+                for shard in self._shards.values():
+                    if tensor_name in shard.entries:
+                        path = self._where[tensor_name] = shard.path
+                        break
         return path is not None and tensor_name in self._shard(path).entries
 
     def tensor(self, tensor_name: str) -> np.ndarray | None:

@@ -84,17 +84,38 @@ _counters: dict = {}
 
 
 def sync_counters(device, n: int) -> torch.Tensor:
-    """int32 array of group counters of the current (device, stream) for the
-    one-launch layer kernel. Zeroed when created; the kernel leaves it zero, so it
-    is reused as is."""
+    """int32 array of group counters / accumulators of the current (device, stream) for
+    the one-launch layer kernel and the MoE chain, at least ``n + 2`` ints. Zeroed when
+    created; the kernels leave it zero, so it is reused as is. Its last int is the
+    status word the library sets when a split reduction gives up
+    (``check_counters`` reads it)."""
     key = _buffer_key(device)
     buf = _counters.get(key)
-    if buf is None or buf.numel() < n:
+    if buf is None or buf.numel() < n + 2:
         if buf is not None:
             _retired.append(buf)
-        buf = torch.zeros(max(int(n), 4096), dtype=torch.int32, device=device)
+        buf = torch.zeros(max(int(n) + 2, 4096), dtype=torch.int32, device=device)
         _counters[key] = buf
     return buf
+
+
+def check_counters(device) -> None:
+    """Waits for the current stream and raises RuntimeError if a split reduction on its
+    counters gave up (``exl3_counters_status``: the array was not zero on entry, or two
+    calls overlapped on it; the affected outputs are NaN) or if the array is not all zero
+    as every finished launch leaves it. Either way the array is zeroed again, so the
+    next call starts clean. A synchronisation: for tests and debugging, not the hot path."""
+    buf = _counters.get(_buffer_key(device))
+    if buf is None:
+        return
+    rc = _lib.load().exl3_counters_status(_ptr(buf), buf.numel(), _stream())
+    dirty = int(buf.ne(0).sum())
+    if rc != _lib.EXL3_OK or dirty:
+        buf.zero_()
+        torch.cuda.current_stream().synchronize()
+        if rc != _lib.EXL3_OK:
+            _lib.check(rc, "exl3_counters_status")
+        raise RuntimeError(f"{dirty} words of the split-reduction counters were left non-zero")
 
 
 def as_trellis_tensor(trellis, device=None) -> torch.Tensor:
@@ -667,7 +688,9 @@ def moe_forward(x2d, indices, gu_trellis, gu_suh, gu_svh, dn_trellis, dn_suh, dn
         _ptr(x2d), T, _ptr(indices), top_k, _ptr(gu_trellis), _ptr(gu_suh), _ptr(gu_svh),
         _ptr(dn_trellis), _ptr(dn_suh), _ptr(dn_svh), E, D, H, int(k), int(cb), int(activation),
         _ptr(y), _ptr(ws), ws.numel(), _ptr(cnt) if cnt is not None else None,
-        n_cnt if cnt is not None else 0, _stream(),  # the length asked for, not the buffer's
+        # the length asked for (it selects the reduction), not the buffer's, plus the two
+        # ints that make the last one the status word
+        n_cnt + 2 if cnt is not None else 0, _stream(),
     )
     _lib.check(rc, "exl3_moe_forward")
     return y

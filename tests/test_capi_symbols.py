@@ -9,8 +9,8 @@ import pytest
 from conftest import ROOT
 
 
-def _declared():
-    text = open(os.path.join(ROOT, "include", "exl3_hip.h")).read()
+def _declared(header="exl3_hip.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(exl3_[a-z0-9_]+)\s*\(", text)))
 
@@ -36,12 +36,25 @@ def test_binding_table_matches_header(lib):
     assert sorted(_lib.PROTOTYPES) == _declared()
 
 
+def test_diag_library_matches_its_header():
+    """The measurement probes live in a library of their own (include/exl3_diag.h) and
+    the product library exports none of them."""
+    from ponyexl3_amd import _lib
+
+    diag = _lib.load_diag()
+    names = _declared("exl3_diag.h")
+    assert names == sorted(_lib.DIAG_PROTOTYPES) and len(names) == 4
+    for n in names:
+        assert hasattr(diag, n)
+        assert not hasattr(_lib.load(), n), f"{n} must not be exported by libexl3_hip.so"
+
+
 def test_version_and_status_strings(lib):
     from ponyexl3_amd import _lib
 
     assert lib.exl3_version() >= 100
     assert _lib.status_string(0) == "ok"
-    for code in range(-8, 0):
+    for code in range(-10, 0):
         assert _lib.status_string(code) not in ("", "unknown status")
     assert lib.exl3_gemv_max_rows() == 8
 

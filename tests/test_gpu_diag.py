@@ -1,4 +1,4 @@
-"""The two diagnostic entry points behind bench.py's measured ceilings: argument
+"""The diagnostic entry points (libexl3_diag.so, include/exl3_diag.h) behind bench.py's measured ceilings: argument
 checks, and that a launch over a small buffer runs to completion and writes only
 inside the output the header describes."""
 import ctypes
@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 def _args(cuda):
     from ponyexl3_amd import _lib
 
-    lib = _lib.load()
+    lib = _lib.load_diag()
     buf = torch.randint(-2**31, 2**31 - 1, (1 << 20,), dtype=torch.int32, device=cuda)  # 4 MiB
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     return _lib, lib, buf, stream

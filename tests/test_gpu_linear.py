@@ -237,6 +237,100 @@ def test_sibling_cache_sees_in_place_updates(cuda):
     assert group._cache_out is None and group._cache_key is None  # both members served
 
 
+def test_bounded_wait_gives_up_visibly(cuda, monkeypatch):
+    """The finishing workgroup of the accumulator reduction waits a bounded number of
+    polls for the other workgroups' adds. With an accumulator pre-seeded so that its
+    count can never come out right and the bound lowered through EXL3_SPIN_LIMIT, every
+    kernel still exits, the affected 128-column group is NaN, the other groups are
+    untouched, exl3_counters_status reports it, and after zeroing the array the next
+    call is right again."""
+    from ponyexl3_amd import make_exl3_layer, ops
+
+    layer = make_exl3_layer(k=4, in_features=1024, out_features=384, seed=97)
+    tr = ops.as_trellis_tensor(layer.trellis, cuda)
+    suh, svh = torch.from_numpy(layer.suh).to(cuda), torch.from_numpy(layer.svh).to(cuda)
+    xt = torch.randn((2, 1024), device=cuda).half()
+    good = ops.linear_forward(xt, tr, 4, 0, suh, svh, fused=True)
+    ops.check_counters(cuda)
+    cnt = ops.sync_counters(cuda, 1)
+    # accumulator of (row 0, column 128 + 5): a count of 255 before anybody has added
+    cnt.view(torch.int64)[128 + 5] = -(1 << 56)
+    monkeypatch.setenv("EXL3_SPIN_LIMIT", "4")
+    print("linear bounded wait", flush=True)
+    bad = ops.linear_forward(xt, tr, 4, 0, suh, svh, fused=True)
+    torch.cuda.synchronize()
+    assert torch.isnan(bad[:, 128:256].float()).all()
+    assert torch.equal(bad[:, :128], good[:, :128]) and torch.equal(bad[:, 256:], good[:, 256:])
+    with pytest.raises(RuntimeError):
+        ops.check_counters(cuda)
+    monkeypatch.delenv("EXL3_SPIN_LIMIT")
+    assert torch.equal(ops.linear_forward(xt, tr, 4, 0, suh, svh, fused=True), good)
+    ops.check_counters(cuda)
+
+
+def test_sibling_cache_under_inference_mode(cuda):
+    """Tensors made under torch.inference_mode() have no version counter; the sibling
+    cache must still work there, and a buffer refilled in place between two steps
+    must not be served the previous step's outputs."""
+    from ponyexl3_amd import EXL3Linear, FusedEXL3Group, make_exl3_layer
+
+    layers = [make_exl3_layer(k=4, in_features=256, out_features=128, seed=95 + i, key=f"i{i}") for i in range(2)]
+    group = FusedEXL3Group(layers)
+    s0, s1 = group.sibling(0), group.sibling(1)
+    with torch.inference_mode():
+        x = torch.randn((1, 256), device=cuda).half()
+        assert x.is_inference()
+        a0, a1 = s0(x).clone(), s1(x).clone()
+        assert torch.equal(a0, EXL3Linear(layers[0])(x)) and torch.equal(a1, EXL3Linear(layers[1])(x))
+        x.copy_(torch.randn((1, 256), device=cuda).half())  # same tensor object, new values
+        b0, b1 = s0(x), s1(x)
+        assert torch.equal(b0, EXL3Linear(layers[0])(x)) and not torch.equal(a0, b0)
+        assert torch.equal(b1, EXL3Linear(layers[1])(x))
+        # a step that asks only one member: the next step's request for it recomputes
+        c0 = s0(x).clone()
+        x.copy_(torch.randn((1, 256), device=cuda).half())
+        d0 = s0(x)
+        assert torch.equal(d0, EXL3Linear(layers[0])(x)) and not torch.equal(c0, d0)
+
+
+CONFIG3_LAUNCHES = [
+    ("qkv", 5120, (8192, 1024, 1024)),
+    ("o_proj", 8192, (5120,)),
+    ("gate_up", 5120, (17408, 17408)),
+    ("down_proj", 17408, (5120,)),
+]
+
+
+@pytest.mark.parametrize("name,n_in,outs", CONFIG3_LAUNCHES)
+def test_config3_whole_layer_against_oracle(cuda, oracle, name, n_in, outs):
+    """M = 2048 through the path a caller uses (ponyexl3/mlx/exl3_linear.py:137-161):
+    rotation, the prefill GEMM (sibling groups as one launch with a per-block member
+    table, split tiles and their completion), output Hadamard and svh, on the four
+    launches of a 27B-class decoder layer. 24 rows spread over the row blocks are
+    compared with the oracle's forward of each member (rel-L2 <= 1e-3)."""
+    from ponyexl3_amd import EXL3Linear, FusedEXL3Group, make_exl3_layer
+
+    members = [make_exl3_layer(k=4, in_features=n_in, out_features=o, seed=30_000 + 10 * i + len(name),
+                               key=f"{name}{i}") for i, o in enumerate(outs)]
+    rng = np.random.default_rng(len(name))
+    x = rng.standard_normal((2048, n_in)).astype(np.float16)
+    xt = torch.from_numpy(x).to(cuda)
+    print(f"config3 layer {name}", flush=True)
+    if len(members) > 1:
+        ys = FusedEXL3Group(members, cuda).forward_all(xt)
+    else:
+        ys = (EXL3Linear(members[0], cuda)(xt),)
+    sample = np.unique(np.concatenate([np.arange(0, 2048, 128), np.arange(2047, 0, -293)]))
+    assert len(sample) >= 16
+    for y, m in zip(ys, members):
+        assert tuple(y.shape) == (2048, m.out_features)
+        ref = oracle.linear_forward(m.trellis, 4, 0, m.suh, m.svh, x[sample])
+        got = y.cpu().numpy()[sample]
+        assert rel_l2(got, ref) <= TOL
+        worst_row = max(rel_l2(got[i], ref[i]) for i in range(len(sample)))
+        assert worst_row <= 2e-3
+
+
 @pytest.mark.parametrize("rows", [1, 3, 8, 13, 16])
 @pytest.mark.parametrize("k,n_in,n_out", [(4, 512, 384), (3, 1024, 256), (6, 2176, 640), (4, 5120, 1024)])
 def test_one_launch_layer_equals_three_launch_chain(cuda, rows, k, n_in, n_out):

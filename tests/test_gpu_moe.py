@@ -241,11 +241,46 @@ def test_moe_equals_linear_modules(cuda):
             assert float((got - ref[0]).abs().max() / (ref.abs().max() + 1e-9)) < 5e-3
 
 
-def test_config4_a3b_shapes(cuda):
+def test_bounded_wait_gives_up_visibly(cuda, monkeypatch):
+    """A counters array that is not zero on entry breaks the accumulator reduction of
+    gate/up: the finishing workgroup's wait for complete counts is bounded (lowered here
+    through EXL3_SPIN_LIMIT so that it runs out at once), every kernel still exits, the
+    slot's output is NaN, the other slots are untouched and the status word is set."""
+    from ponyexl3_amd import EXL3SwitchGLU, ops
+
+    E, D, H, kk, k = 4, 640, 256, 2, 4
+    gate, up, down = _experts(E, D, H, k, False, 900)
+    moe = EXL3SwitchGLU.from_layers(gate, up, down)
+    rng = np.random.default_rng(9)
+    xt = torch.from_numpy((rng.standard_normal((1, D)) * 0.5).astype(np.float16)).to(cuda)
+    it = torch.tensor([[2, 1]], dtype=torch.int32, device=cuda)
+    args = (xt, it, moe._gu_trellis, moe._gu_suh, moe._gu_svh, moe._dn_trellis, moe._dn_suh, moe._dn_svh,
+            k, moe._cb)
+    good = ops.moe_forward(*args, fused=True)
+    ops.check_counters(cuda)
+    cnt = ops.sync_counters(cuda, 1)
+    # accumulator of (slot 0, gate, column 5): a count of 255 that can never come out right
+    cnt.view(torch.int64)[5] = -(1 << 56)
+    monkeypatch.setenv("EXL3_SPIN_LIMIT", "4")
+    print("moe bounded wait", flush=True)
+    bad = ops.moe_forward(*args, fused=True)
+    torch.cuda.synchronize()
+    assert torch.isnan(bad[0, 0].float()).all()
+    assert torch.equal(bad[0, 1], good[0, 1])
+    with pytest.raises(RuntimeError):
+        ops.check_counters(cuda)
+    monkeypatch.delenv("EXL3_SPIN_LIMIT")
+    assert torch.equal(ops.moe_forward(*args, fused=True), good)  # check_counters zeroed the array
+    ops.check_counters(cuda)
+
+
+def test_config4_a3b_shapes(cuda, oracle):
     """hidden 2048, 256 experts of 2048->512 / 512->2048, top-8 routing from a
-    softmax over seeded router logits, at 1 and 8 tokens. The result is checked
-    against per-expert EXL3Linear chains of the same (oracle-checked) kernels on
-    a sample of slots, and permutation equivariance over the slot order."""
+    softmax over seeded router logits, at 1 and 8 tokens. Every (token, expert) slot
+    is checked against the oracle's unfused expert chain
+    (ponyexl3/mlx/exl3_moe.py:648-682) at rel-L2 <= 1e-3, two slots also against
+    per-expert EXL3Linear chains, and the slot order against permutation
+    equivariance."""
     from ponyexl3_amd import EXL3Layer, EXL3Linear, EXL3SwitchGLU, ops
     from ponyexl3_amd.moe import combine_experts, route_topk
 
@@ -274,8 +309,24 @@ def test_config4_a3b_shapes(cuda):
         perm = torch.randperm(kk, generator=torch.Generator().manual_seed(T)).to(cuda)
         y2 = moe(xt.reshape(1, T, D), inds[:, perm].reshape(1, T, kk))
         assert torch.equal(y2, y[:, :, perm])
-        # two sampled slots against stand-alone layers cut out of the stacks
+        # all T * 8 slots against the oracle's chain over the selected experts
         gt = H // 16
+        cut = lambda a: np.ascontiguousarray(a)
+        experts = {}
+        for e in sorted(set(int(v) for v in inds.cpu().numpy().ravel())):
+            experts[e] = {
+                "gate": (cut(gu[:, e * gt : (e + 1) * gt]), gu_suh[e, 0], gu_svh[e, :H]),
+                "up": (cut(gu[:, (E + e) * gt : (E + e + 1) * gt]), gu_suh[e, 1], gu_svh[e, H:]),
+                "down": (cut(dn[:, e * (D // 16) : (e + 1) * (D // 16)]), dn_suh[e], dn_svh[e]),
+            }
+        ref_all = oracle.moe_experts_forward(experts, x, inds.cpu().numpy(), k, 0)
+        got_all = y[0].cpu().numpy()
+        worst = max(float(np.linalg.norm(got_all[t, s].astype(np.float64) - ref_all[t, s].astype(np.float64))
+                          / np.linalg.norm(ref_all[t, s].astype(np.float64)))
+                    for t in range(T) for s in range(kk))
+        print(f"config4 T={T}: worst slot rel-L2 vs oracle {worst:.2e}", flush=True)
+        assert worst <= 1e-3
+        # two sampled slots against stand-alone layers cut out of the stacks
         for (t, s) in [(0, 0), (T - 1, kk - 1)]:
             e = int(inds[t, s])
             mk = lambda tr, suh, svh, n_in, n_out: EXL3Linear(

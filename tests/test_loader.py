@@ -149,3 +149,57 @@ def test_directory_is_scanned_once_and_shards_found_without_an_index(tmp_path):
     assert meta.as_dict()["trellis_shape"] == (8, 8, 96)
     ck = loader.open_checkpoint(d)
     assert ck is loader.open_checkpoint(d) and ck.tensor("no.such.tensor") is None
+
+
+def test_index_that_omits_tensors_and_corrupt_headers(tmp_path):
+    """An index that lists the trellis but not the scales, bias or multiplier of a layer:
+    the shards are looked through once and the layer still loads complete
+    (ponyexl3/ref/loader.py:108-125 searches the shards per tensor). Offsets or a header
+    length that point outside the file are refused."""
+    import struct
+
+    layers = _layers()
+    d = _write_checkpoint(tmp_path, layers, shards=2)
+    index_path = os.path.join(d, "model.safetensors.index.json")
+    weight_map = json.load(open(index_path))["weight_map"]
+    kept = {n: f for n, f in weight_map.items() if n.endswith(".trellis")}
+    assert len(kept) < len(weight_map)
+    json.dump({"weight_map": kept}, open(index_path, "w"))
+    loader.clear_weight_index_cache(d)
+    for l in layers:
+        got = loader.load_exl3_layer(d, l.key)
+        np.testing.assert_array_equal(got.suh, l.suh)
+        np.testing.assert_array_equal(got.svh, l.svh)
+        assert (got.bias is None) == (l.bias is None)
+    # the multiplier check still runs for tensors the index does not list
+    d2 = tmp_path / "wrong"
+    d2.mkdir()
+    d2 = _write_checkpoint(d2, layers, shards=2, wrong_mcg=layers[0].key)
+    wm = json.load(open(os.path.join(d2, "model.safetensors.index.json")))["weight_map"]
+    json.dump({"weight_map": {n: f for n, f in wm.items() if not n.endswith(".mcg")}},
+              open(os.path.join(d2, "model.safetensors.index.json"), "w"))
+    loader.clear_weight_index_cache(d2)
+    with pytest.raises(ValueError, match="multiplier"):
+        loader.load_exl3_layer(d2, layers[0].key)
+
+    # data offsets beyond the file
+    d3 = tmp_path / "corrupt"
+    d3.mkdir()
+    d3 = _write_checkpoint(d3, layers[:1])
+    path = os.path.join(d3, "model.safetensors")
+    raw = open(path, "rb").read()
+    (hlen,) = struct.unpack("<Q", raw[:8])
+    header = json.loads(raw[8 : 8 + hlen])
+    name = layers[0].key + ".trellis"
+    lo, hi = header[name]["data_offsets"]
+    header[name]["data_offsets"] = [lo + (1 << 30), hi + (1 << 30)]
+    blob = json.dumps(header).encode()
+    open(path, "wb").write(struct.pack("<Q", len(blob)) + blob + raw[8 + hlen :])
+    loader.clear_weight_index_cache(d3)
+    with pytest.raises(ValueError, match="outside"):
+        loader.load_exl3_layer(d3, layers[0].key)
+    # header length beyond the file
+    open(path, "wb").write(struct.pack("<Q", 1 << 40) + blob)
+    loader.clear_weight_index_cache(d3)
+    with pytest.raises(ValueError, match="past the end"):
+        loader.load_exl3_layer(d3, layers[0].key)
