@@ -22,7 +22,7 @@ extern "C" {
  *   loads; out: 4 bytes of device memory, practically never written.
  * exl3_diag_decode_loop: n_wg workgroups of 16 waves run `steps` (a multiple of 4)
  *   iterations of the small-batch kernels' inner loop (one wave-wide load of 256*K
- *   bytes, per-lane decode of 32 codewords, 8 matrix-pipe dot products) over
+ *   bytes, per-lane decode of 32 codewords, 16 matrix-pipe dot products) over
  *   consecutive 256*K-byte rows of buf, wrapping at the largest power-of-two row
  *   count that fits in `bytes`; weights per launch = n_wg*16*steps*2048. cb 0 or 1.
  *   out: float [n_wg*1024].

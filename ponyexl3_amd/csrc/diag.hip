@@ -37,14 +37,16 @@ template <int K, int CB>
 __global__ __launch_bounds__(1024) void diag_decode_kernel(const uint32_t* __restrict__ buf,
                                                            uint32_t rows_mask, int steps,
                                                            float* __restrict__ out) {
-    __shared__ __attribute__((aligned(16))) half_t xs[1024];
+    // 64 tile rows of activations, each value stored twice as the layer kernels stage them
+    __shared__ __attribute__((aligned(16))) half_t xs[2048];
     constexpr int kSlots = 4;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    xs[threadIdx.x] = (half_t)(float)((int)(threadIdx.x * 37 % 17) - 8);  // small integers, -8..8
+    const half_t xval = (half_t)(float)((int)(threadIdx.x * 37 % 17) - 8);  // small integers, -8..8
+    xs[2 * threadIdx.x] = xs[2 * threadIdx.x + 1] = xval;
     __syncthreads();
     const uint32_t wave_global = blockIdx.x * 16 + wave;
-    float4_t accv[2] = {float4_t{0, 0, 0, 0}, float4_t{0, 0, 0, 0}};
+    float4_t accv[2][1] = {{float4_t{0, 0, 0, 0}}, {float4_t{0, 0, 0, 0}}};
     uint32_t w[kSlots][K];
     auto row_ptr = [&](int s) {
         const uint32_t r = (wave_global * (uint32_t)steps + (uint32_t)s) & rows_mask;
@@ -57,31 +59,20 @@ __global__ __launch_bounds__(1024) void diag_decode_kernel(const uint32_t* __res
 #pragma unroll
         for (int s = 0; s < kSlots; s++) {
             const uint32_t prev_next = neighbour_word(w[(s + 1) % kSlots][K - 1], lane);
-            const uint4_t* xp = reinterpret_cast<const uint4_t*>(xs + ((s0 + s) & 63) * 16);
-            const uint4_t x0 = xp[0], x1 = xp[1];
+            const uint4_t* xp = reinterpret_cast<const uint4_t*>(xs + ((s0 + s) & 63) * 32);
             __builtin_amdgcn_sched_barrier(0);
-            const LaneWords<K> lw = make_lane_words<K>(prev, w[s]);
-            half2_t wp[16];
-            decode_lane<K, CB>(lw, wp);
-#pragma unroll
-            for (int j4 = 0; j4 < 4; j4++) {
-                const uint4_t xv = (j4 >> 1) ? x1 : x0;
-                const uint2_t xa = (j4 & 1) ? uint2_t{xv.z, xv.w} : uint2_t{xv.x, xv.y};
-#pragma unroll
-                for (int cs = 0; cs < 2; cs++) {
-                    const uint2_t wb = {half2_to_bits(wp[8 * cs + 2 * j4]),
-                                        half2_to_bits(wp[8 * cs + 2 * j4 + 1])};
-                    accv[cs] = __builtin_amdgcn_mfma_f32_4x4x4f16(
-                        __builtin_bit_cast(half4_t, xa), __builtin_bit_cast(half4_t, wb), accv[cs], 0,
-                        0, 0);
-                }
-            }
+            dot_tile_row<K, CB, 1>(make_lane_words<K>(prev, w[s]), [&](int c) {
+                XChunk<1> t;
+                t.v[0] = xp[c];
+                return t;
+            }, accv);
             load_lane_words_nt<K>(row_ptr(s0 + s + kSlots), w[s]);
             __builtin_amdgcn_sched_barrier(0);
             prev = prev_next;
         }
     }
-    out[(size_t)wave_global * 64 + lane] = accv[0][0] + accv[1][0];
+    const float total = accv[0][0][0] + accv[1][0][0];
+    out[(size_t)wave_global * 64 + lane] = total;
 }
 
 // The fixed phases of a small-batch launch, measured on a grid of the caller's choice:

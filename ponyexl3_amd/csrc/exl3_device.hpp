@@ -143,6 +143,17 @@ __device__ __forceinline__ void decode_pair2(uint32_t cw0, uint32_t cw1, uint32_
     }
 }
 
+// One codeword -> the dword whose two fp16 halves add up to the weight (3INST / MCG:
+// the scrambled word itself; MUL1: the weight and a zero). A dot product is linear, so
+// a kernel that feeds both halves to the matrix pipe as two k-slots against the same
+// activation gets a * lo + a * hi in fp32 - the product with the exact sum of the two
+// halves, which the fp16 weight is the rounding of - and saves the half add.
+template <int CB>
+__device__ __forceinline__ uint32_t weight_halves(uint32_t cw) {
+    if constexpr (CB == CB_MUL1) return (uint32_t)half_to_bits(decode_mul1(cw));
+    else return scramble<CB>(cw);
+}
+
 // The K+1 dwords a lane needs for its 32 codewords: w[0] is the dword that
 // precedes the lane's own K dwords (already wrapped), w[1..K] are its own.
 template <int K>
@@ -220,6 +231,78 @@ __device__ __forceinline__ void decode_lane(const LaneWords<K>& lw, half2_t (&wp
         decode_pair2<CB>(lane_codeword<K, na>(lw), lane_codeword<K, na + 1>(lw),
                          lane_codeword<K, nb>(lw), lane_codeword<K, nb + 1>(lw), wp[ia], wp[ib]);
     });
+}
+
+// Cross-lane butterflies of the Walsh-Hadamard transforms, without a trip through LDS.
+// Stage "lane ^ 2^BIT" of a value held one per lane: the lane whose BIT is clear gets
+// v + partner, the other one partner - v. For BIT 0..3 the partner comes through a DPP
+// operand (quad permutations for 1 and 2, a quad reversal followed by a half-row mirror
+// for 4, a row rotation by 8 for 8) and the subtraction is the addition of v with its
+// sign flipped in the upper lanes (`sign` = lane_sign_mask(lane, BIT)): partner + (-v)
+// and v + partner round exactly like partner - v and v + partner.
+__device__ __forceinline__ uint32_t lane_sign_mask(int lane, int bit) {
+    return ((uint32_t)lane << (31 - bit)) & 0x80000000u;
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+
+template <int BIT>
+__device__ __forceinline__ float butterfly_dpp(float v, uint32_t sign) {
+    static_assert(BIT >= 0 && BIT <= 3, "lanes 16 and 32 apart are reached by swapping registers");
+    const float own = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v) ^ sign);
+    float partner;
+    if constexpr (BIT == 0) partner = dpp_move<0xB1>(v);                         // quad_perm [1,0,3,2]
+    else if constexpr (BIT == 1) partner = dpp_move<0x4E>(v);                    // quad_perm [2,3,0,1]
+    else if constexpr (BIT == 2) partner = dpp_move<0x141>(dpp_move<0x1B>(v));   // [3,2,1,0], row_half_mirror
+    else partner = dpp_move<0x128>(v);                                           // row_ror:8
+    return __fadd_rn(partner, own);
+}
+
+// Stages "lane ^ 16" and "lane ^ 32" for two values a, b that both need them: the swap
+// instructions of gfx950 exchange the odd 16-lane rows (upper 32 lanes) of a with the
+// even rows (lower 32 lanes) of b, after which every lane holds a value and its partner
+// side by side (even rows / lower half: those of a; the others: those of b), and the
+// stage is an add and a subtract inside the lane. swap_back restores the layout (both
+// swaps are involutions; undo them in reverse order).
+__device__ __forceinline__ void swap_rows16(float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap_halves32(float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void butterfly_in_lane(float& a, float& b) {
+    const float s = __fadd_rn(a, b), d = __fsub_rn(a, b);
+    a = s;
+    b = d;
+}
+
+// Unnormalised WHT over 128 values held as (a, b) = elements (2*lane, 2*lane+1);
+// same butterfly order as ponyexl3/ref/hadamard.py:16-30 (stage h pairs i, i+h): inside
+// the lane, then lanes 1, 2, 4, 8 apart through DPP operands, then 16 and 32 apart by
+// swapping registers. No LDS traffic and no waits: a wave that has its activations
+// starts decoding a few dozen instructions later.
+__device__ __forceinline__ void wht128_lanes(float& a, float& b, int lane) {
+    butterfly_in_lane(a, b);
+    const uint32_t s0 = lane_sign_mask(lane, 0), s1 = lane_sign_mask(lane, 1),
+                   s2 = lane_sign_mask(lane, 2), s3 = lane_sign_mask(lane, 3);
+    a = butterfly_dpp<0>(a, s0);
+    b = butterfly_dpp<0>(b, s0);
+    a = butterfly_dpp<1>(a, s1);
+    b = butterfly_dpp<1>(b, s1);
+    a = butterfly_dpp<2>(a, s2);
+    b = butterfly_dpp<2>(b, s2);
+    a = butterfly_dpp<3>(a, s3);
+    b = butterfly_dpp<3>(b, s3);
+    swap_rows16(a, b);
+    butterfly_in_lane(a, b);
+    swap_halves32(a, b);
+    butterfly_in_lane(a, b);
+    swap_halves32(a, b);
+    swap_rows16(a, b);
 }
 
 __device__ __forceinline__ float dot2(half2_t a, half2_t b, float c) {

@@ -11,10 +11,87 @@ namespace exl3 {
 
 constexpr float kHadScaleF = 0.088388347648318440550f;  // 1/sqrt(128)
 
-// Row stride (halfs) of a wave's staged activation block [MT][kXwLd]: 128 values
-// plus 16 bytes, so that the four batch rows a quad of lanes reads with one
-// ds_read_b128 start four LDS banks apart instead of in the same bank.
-constexpr int kXwLd = 136;
+// Row stride (halfs) of a wave's staged activation block [MT][kXwLd]: the 128 values of
+// a block, each stored twice in a row (x0, x0, x1, x1, ...: the matrix-pipe operand
+// that meets the unsummed halves of the weights), plus 16 bytes, so that the four batch
+// rows a quad of lanes reads with one ds_read_b128 start four LDS banks apart instead
+// of in the same bank.
+constexpr int kXwLd = 264;
+
+// Activations of a tile row as the matrix pipe takes them, a quarter at a time: for each
+// group of four batch rows, lane i of every quad reads batch row 4q+i; chunk c = input
+// rows 4c..4c+3 of the tile row, each value twice (one ds_read_b128).
+template <int MT>
+struct XChunk {
+    uint4_t v[(MT + 3) / 4];
+};
+
+template <int MT>
+__device__ __forceinline__ XChunk<MT> load_x_chunk(half_t (*xw)[kXwLd], int row_in_block, int xlane,
+                                                   int c) {
+    constexpr int NQ = (MT + 3) / 4;
+    XChunk<MT> t;
+#pragma unroll
+    for (int q = 0; q < NQ; q++) {
+        int m = 4 * q + xlane;
+        if (m > MT - 1) m = MT - 1;  // rows past the batch repeat a staged row; never used
+        t.v[q] = *reinterpret_cast<const uint4_t*>(&xw[m][row_in_block * 32 + 8 * c]);
+    }
+    return t;
+}
+
+// The dot products of one tile row on the matrix pipe: v_mfma_f32_4x4x4_16b_f16
+// multiplies, in each of its 16 independent blocks of 4 lanes, a 4x4 A (lane i of the
+// block supplies row i) with a 4x4 B (lane j supplies column j) and leaves D[0..3][j] in
+// lane j. A row i = activations of batch row 4q+i, B column j = two consecutive weights
+// of lane j's own output column as their unsummed halves (lo, hi, lo', hi') against
+// (a, a, a', a'): every lane gets the dot products of its weights with four batch rows,
+// no data crosses lanes, and the VALU only extracts, multiplies and masks.
+//
+// Order of work: the sixteen codeword pairs of a lane are taken chunk by chunk of the
+// activations (input rows 0-3, 8-11, 4-7, 12-15 of the tile row, both columns each), so
+// that only two chunks are live at a time: the third and fourth are requested from LDS
+// when the first and second have been used up. The matrix instruction of a pair is
+// issued after the next pair has been decoded, so it never waits for the VALU result
+// it reads.
+template <int K, int CB, int MT, class LoadChunk>
+__device__ __forceinline__ void dot_tile_row(const LaneWords<K>& lw, LoadChunk&& load_chunk,
+                                             float4_t (&accv)[2][(MT + 3) / 4]) {
+    constexpr int NQ = (MT + 3) / 4;
+    // pair t: column select cs = (t >> 1) & 1 ... see pair_n below
+    // t = 4*phase + 2*jj + cs with chunk(phase) = {0, 2, 1, 3}[phase], j = 2*chunk + jj
+    auto pair_j = [](int t) constexpr { return 2 * ((t >> 2) == 0 ? 0 : (t >> 2) == 1 ? 2 : (t >> 2) == 2 ? 1 : 3) + ((t >> 1) & 1); };
+    auto pair_cs = [](int t) constexpr { return t & 1; };
+    // codewords n, n+1 hold input rows 2j, 2j+1 of column u + 8*cs (cw_row, cw_col_sel)
+    auto pair_n = [](int j, int cs) constexpr { return 8 * (j & 3) + 4 * cs + 2 * (j >> 2); };
+    XChunk<MT> xc[4];
+    xc[0] = load_chunk(0);
+    xc[2] = load_chunk(2);
+    uint2_t wb[16];
+    auto issue = [&](auto tc) {
+        constexpr int t = tc.value;
+        constexpr int j = pair_j(t), cs = pair_cs(t);
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            const uint4_t xv = xc[j >> 1].v[q];
+            const uint2_t xa = (j & 1) ? uint2_t{xv.z, xv.w} : uint2_t{xv.x, xv.y};
+            accv[cs][q] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4_t, xa),
+                                                           __builtin_bit_cast(half4_t, wb[t]),
+                                                           accv[cs][q], 0, 0, 0);
+        }
+    };
+    static_for<0, 16>([&](auto tc) {
+        constexpr int t = tc.value;
+        constexpr int n = pair_n(pair_j(t), pair_cs(t));
+        static_assert(cw_col_sel(n) == pair_cs(t) && (cw_row(n) >> 1) == pair_j(t), "pair order");
+        wb[t] = uint2_t{weight_halves<CB>(lane_codeword<K, n>(lw)),
+                        weight_halves<CB>(lane_codeword<K, n + 1>(lw))};
+        if constexpr (t >= 1) issue(std::integral_constant<int, t - 1>{});
+        if constexpr (t == 4) xc[1] = load_chunk(1);   // chunk 0 has just been used up
+        if constexpr (t == 8) xc[3] = load_chunk(3);   // chunk 2 likewise
+    });
+    issue(std::integral_constant<int, 15>{});
+}
 
 template <int K>
 __device__ __forceinline__ void load_lane_words_nt(const uint32_t* __restrict__ p,
@@ -31,23 +108,6 @@ template <int K>
 __device__ __forceinline__ void load_lane_words_nt(global_words_t p, uint32_t (&own)[K]) {
 #pragma unroll
     for (int i = 0; i < K; i++) own[i] = __builtin_nontemporal_load(p + i);
-}
-
-// Unnormalised WHT over 128 values held as (a, b) = elements (2*lane, 2*lane+1);
-// same butterfly order as ponyexl3/ref/hadamard.py:16-30 (stage h pairs i, i+h).
-__device__ __forceinline__ void wht128_lanes(float& a, float& b, int lane) {
-    const float s = a + b, d = a - b;
-    a = s;
-    b = d;
-#pragma unroll
-    for (int bit = 0; bit < 6; bit++) {
-        const int mask = 1 << bit;
-        const float pa = __shfl_xor(a, mask, kWave);
-        const float pb = __shfl_xor(b, mask, kWave);
-        const bool upper = (lane & mask) != 0;
-        a = upper ? pa - a : a + pa;
-        b = upper ? pb - b : b + pb;
-    }
 }
 
 // One wave streams tile rows [tk_begin, tk_end) (both multiples of 8, non-empty)
@@ -116,61 +176,29 @@ __device__ __forceinline__ void stream_block_rows_at(const uint32_t* __restrict_
                 o.x = (half_t)__fmul_rn(a, kHadScaleF);
                 o.y = (half_t)__fmul_rn(b, kHadScaleF);
             }
-            *reinterpret_cast<half2_t*>(&xw[m][2 * lane]) = o;
+            const uint32_t lo = half_to_bits(o.x), hi = half_to_bits(o.y);
+            *reinterpret_cast<uint2_t*>(&xw[m][4 * lane]) = uint2_t{lo | (lo << 16), hi | (hi << 16)};
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
     };
-    // The dot products run on the matrix pipe, which works in the shadow of the
-    // decode VALU stream: v_mfma_f32_4x4x4_16b_f16 multiplies, in each of its 16
-    // independent blocks of 4 lanes, a 4x4 A (lane i of the block supplies row i)
-    // with a 4x4 B (lane j supplies column j) and leaves D[0..3][j] in lane j.
-    // With A row i = activations of batch row 4q+i and B column j = four
-    // consecutive weights of lane j's own output column, every lane gets the dot
-    // products of its weights with four batch rows; no data crosses lanes.
     constexpr int NQ = (MT + 3) / 4;  // groups of four batch rows
     float4_t accv[2][NQ];
 #pragma unroll
     for (int cs = 0; cs < 2; cs++)
 #pragma unroll
         for (int q = 0; q < NQ; q++) accv[cs][q] = float4_t{0.f, 0.f, 0.f, 0.f};
-    struct XTile {
-        uint4_t q[NQ][2];
-    };
     const int xlane = lane & 3;
-    auto load_x = [&](int row_in_block) {
-        XTile t;
-#pragma unroll
-        for (int q = 0; q < NQ; q++) {
-            int m = 4 * q + xlane;
-            if (m > MT - 1) m = MT - 1;  // rows past the batch repeat a staged row; never used
-            const uint4_t* xp = reinterpret_cast<const uint4_t*>(&xw[m][row_in_block * 16]);
-            t.q[q][0] = xp[0];
-            t.q[q][1] = xp[1];
-        }
-        return t;
+    auto consume = [&](const uint32_t (&words)[K], uint32_t prev, int row_in_block) {
+        dot_tile_row<K, CB, MT>(
+            make_lane_words<K>(prev, words),
+            [&](int c) { return load_x_chunk<MT>(xw, row_in_block, xlane, c); }, accv);
     };
-    auto consume = [&](const uint32_t (&words)[K], uint32_t prev, const XTile& xt) {
-        const LaneWords<K> lw = make_lane_words<K>(prev, words);
-        half2_t wp[16];
-        decode_lane<K, CB>(lw, wp);
-        // fresh-row groups outermost: consecutive MFMAs then write 2*NQ different
-        // accumulators, so none waits for the one just issued
+    auto add_up = [&]() {
 #pragma unroll
-        for (int j4 = 0; j4 < 4; j4++) {  // input rows 4*j4 .. 4*j4+3 of the tile
-#pragma unroll
-            for (int q = 0; q < NQ; q++) {
-                const uint4_t xv = xt.q[q][j4 >> 1];
-                const uint2_t xa = (j4 & 1) ? uint2_t{xv.z, xv.w} : uint2_t{xv.x, xv.y};
-#pragma unroll
-                for (int cs = 0; cs < 2; cs++) {
-                    const uint2_t wb = {half2_to_bits(wp[8 * cs + 2 * j4]),
-                                        half2_to_bits(wp[8 * cs + 2 * j4 + 1])};
-                    accv[cs][q] = __builtin_amdgcn_mfma_f32_4x4x4f16(
-                        __builtin_bit_cast(half4_t, xa), __builtin_bit_cast(half4_t, wb),
-                        accv[cs][q], 0, 0, 0);
-                }
-            }
+        for (int m = 0; m < MT; m++) {
+            acc[m][0] += accv[0][m >> 2][m & 3];
+            acc[m][1] += accv[1][m >> 2][m & 3];
         }
     };
     constexpr int kSlots = kStreamSlots;
@@ -189,17 +217,12 @@ __device__ __forceinline__ void stream_block_rows_at(const uint32_t* __restrict_
         for (int s = 0; s < kSlots; s++) {
             const uint32_t prev_next =
                 s + 1 < kSlots ? neighbour_word(buf[s + 1][K - 1], lane) : 0u;
-            const XTile xt = load_x(row0 + s);
             __builtin_amdgcn_sched_barrier(0);
-            consume(buf[s], prev, xt);
+            consume(buf[s], prev, row0 + s);
             __builtin_amdgcn_sched_barrier(0);
             prev = prev_next;
         }
-#pragma unroll
-        for (int m = 0; m < MT; m++) {
-            acc[m][0] += accv[0][m >> 2][m & 3];
-            acc[m][1] += accv[1][m >> 2][m & 3];
-        }
+        add_up();
         return;
     }
     // Ranges are whole blocks, so the staging sits outside the unrolled 8-step
@@ -216,9 +239,8 @@ __device__ __forceinline__ void stream_block_rows_at(const uint32_t* __restrict_
             const int tk = tkb + s8;
             const int slot = s8 & (kSlots - 1);
             const uint32_t prev_next = neighbour_word(buf[(slot + 1) & (kSlots - 1)][K - 1], lane);
-            const XTile xt = load_x(s8);
             __builtin_amdgcn_sched_barrier(0);
-            consume(buf[slot], prev, xt);
+            consume(buf[slot], prev, s8);
             const int tn = min(tk + kSlots, tk_end - 1);
             load_lane_words_nt<K>(base + (size_t)tn * row_words, buf[slot]);
             __builtin_amdgcn_sched_barrier(0);
@@ -226,11 +248,7 @@ __device__ __forceinline__ void stream_block_rows_at(const uint32_t* __restrict_
         }
         tkb += 8;
     } while (tkb < tk_end);
-#pragma unroll
-    for (int m = 0; m < MT; m++) {
-        acc[m][0] += accv[0][m >> 2][m & 3];
-        acc[m][1] += accv[1][m >> 2][m & 3];
-    }
+    add_up();
 }
 
 // The same over `rows` consecutive rows of a row-major activation matrix.

@@ -438,15 +438,17 @@ __global__ __launch_bounds__(256) void gemm_fixup_post_kernel(
                 }
             }
         }
+        // lanes 1, 2, 4, 8 apart through DPP operands, 16 apart by swapping registers
+        static_for<0, 4>([&](auto bit) {
+            const uint32_t sign = lane_sign_mask(lane, bit.value);
 #pragma unroll
-        for (int bit = 0; bit < 5; bit++) {
-            const int mask = 1 << bit;
-            const bool upper = (lane & mask) != 0;
+            for (int j = 0; j < 4; j++) v[j] = butterfly_dpp<bit.value>(v[j], sign);
+        });
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const float q = __shfl_xor(v[j], mask, kWave);
-                v[j] = upper ? __fsub_rn(q, v[j]) : __fadd_rn(v[j], q);
-            }
+        for (int j = 0; j < 4; j += 2) {
+            swap_rows16(v[j], v[j + 1]);
+            butterfly_in_lane(v[j], v[j + 1]);
+            swap_rows16(v[j], v[j + 1]);
         }
         if (col_ok) {
             half_t o[4];

@@ -197,7 +197,13 @@ __global__ __launch_bounds__(NW * 64) void linear_small_kernel(
     const int* __restrict__ group_sub, int in_tiles, int out_tiles, int rows, int n_groups,
     int tk_per_split, int n_splits, int* status, int spin_limit) {
     static_assert(NW == 4 || (NW == 8 && ATOMIC), "eight-wave workgroups use the accumulators");
-    __shared__ __attribute__((aligned(16))) half_t xs[NW][MT][kXwLd];
+    // the staged activations and, once every wave has left the streaming loop, the waves'
+    // sums share one LDS buffer (at eight rows the two together would cost occupancy)
+    constexpr size_t kXsBytes = sizeof(half_t) * NW * MT * kXwLd;
+    constexpr size_t kRedBytes = sizeof(float) * NW * MT * 128;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[kXsBytes > kRedBytes ? kXsBytes : kRedBytes];
+    half_t (*xs)[MT][kXwLd] = reinterpret_cast<half_t (*)[MT][kXwLd]>(smem);
+    float (*red)[MT][128] = reinterpret_cast<float (*)[MT][128]>(smem);
     const int g = blockIdx.x;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -243,8 +249,8 @@ __global__ __launch_bounds__(NW * 64) void linear_small_kernel(
     // counts are complete - a wait for memory operations that are already in flight,
     // not for another wave to be scheduled. Accumulators must be zero on entry; the
     // finisher zeroes them again.
-    __shared__ float red[NW][MT][128];
     const int c0 = (lane >> 3) * 16 + (lane & 7);
+    __syncthreads();  // nobody reads staged activations any more
 #pragma unroll
     for (int m = 0; m < MT; m++) {
         red[wave][m][c0] = acc[m][0];

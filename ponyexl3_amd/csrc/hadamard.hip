@@ -23,20 +23,7 @@ namespace exl3 {
 
 constexpr float kHadScale = 0.088388347648318440550f;  // 1/sqrt(128)
 
-__device__ __forceinline__ void wht128(float& a, float& b, int lane) {
-    const float s = a + b, d = a - b;
-    a = s;
-    b = d;
-#pragma unroll
-    for (int bit = 0; bit < 6; bit++) {
-        const int mask = 1 << bit;
-        const float pa = __shfl_xor(a, mask, kWave);
-        const float pb = __shfl_xor(b, mask, kWave);
-        const bool upper = (lane & mask) != 0;
-        a = upper ? pa - a : a + pa;
-        b = upper ? pb - b : b + pb;
-    }
-}
+__device__ __forceinline__ void wht128(float& a, float& b, int lane) { wht128_lanes(a, b, lane); }
 
 // Optional row gathers / scatter of the wide kernels: kernel row r reads input row
 // in_index[r], scale vector scale_index[r] (scale_ld elements apart) and writes
@@ -74,16 +61,12 @@ __device__ __forceinline__ void wht128_wide(float (&v)[8], int lane) {
             }
         }
     }
+    // lanes 1, 2, 4, 8 apart: DPP operands, no LDS
+    static_for<0, 4>([&](auto bit) {
+        const uint32_t sign = lane_sign_mask(lane, bit.value);
 #pragma unroll
-    for (int bit = 0; bit < 4; bit++) {
-        const int mask = 1 << bit;
-        const bool upper = (lane & mask) != 0;
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const float p = __shfl_xor(v[j], mask, kWave);
-            v[j] = upper ? p - v[j] : v[j] + p;
-        }
-    }
+        for (int j = 0; j < 8; j++) v[j] = butterfly_dpp<bit.value>(v[j], sign);
+    });
 }
 
 __device__ __forceinline__ void halfs_to_floats(uint4_t q, float (&v)[8]) {
