@@ -263,6 +263,10 @@ __global__ __launch_bounds__(NW * 64) void linear_small_kernel(
         const size_t out_total = (size_t)n_groups * 128;
         const int wg_splits = (n_splits + NW - 1) / NW;  // partial rows per group
         const size_t col = (size_t)g * 128 + 2 * lane;
+        // requested now, needed only by the finishing workgroup: by then they are here
+        half2_t sv, bv;
+        if (svh) sv = *reinterpret_cast<const half2_t*>(svh + col);
+        if (bias) bv = *reinterpret_cast<const half2_t*>(bias + col);
         unsigned long long w0[MT], w1[MT];
 #pragma unroll
         for (int m = 0; m < MT; m++) {
@@ -316,9 +320,6 @@ __global__ __launch_bounds__(NW * 64) void linear_small_kernel(
                 if (m < rows) *reinterpret_cast<half2_t*>(y + (size_t)m * out_total + col) = bad;
             return;
         }
-        half2_t sv, bv;
-        if (svh) sv = *reinterpret_cast<const half2_t*>(svh + col);
-        if (bias) bv = *reinterpret_cast<const half2_t*>(bias + col);
 #pragma unroll
         for (int m = 0; m < MT; m++) {
             if (m < rows) {
@@ -481,10 +482,23 @@ GemvPlan plan_linear_small(int rows, int in_tiles, int n_groups, int K) {
     static const int kHalfBelow = env_int("EXL3_LINEAR_HALF_BELOW", 4096, 0, 1 << 20);
     const int target_waves = 256 * 4 * kWavesPerSimd;
     const int n_blocks = in_tiles / 8;
-    // (not with more than 48 blocks: 100+ partial rows per column group cost the
-    // finishing workgroup more than the extra waves gain; measured on 8192 -> 5120)
-    if (rows <= 2 && n_blocks <= 48 && (long long)n_blocks * n_groups < kHalfBelow)
-        return GemvPlan{n_blocks * 2, 4};
+    // Half blocks double the waves, which evens out the load of the SIMDs when whole
+    // blocks leave only a few waves on each (8192 -> 5120: 2560 whole-block waves are
+    // two on half of the 1024 SIMDs and three on the others; 5120 half-block waves are
+    // five everywhere), at the price of rotating every block twice. Cost per SIMD in
+    // issue slots: (most waves on a SIMD) x (tile rows x 118 + 60 for the rotation).
+    // The accumulator reduction has to be able to take the partial sums (eight-bit
+    // count, atomics limit); with partial rows, 100+ rows per column group would cost
+    // the finishing workgroup more than the balance gains.
+    if (rows <= 2 && (long long)n_blocks * n_groups < kHalfBelow) {
+        const long long whole = (long long)n_blocks * n_groups, n_simd = 1024;
+        const long long cost_whole = ((whole + n_simd - 1) / n_simd) * (8 * 118 + 60);
+        const long long cost_half = ((2 * whole + n_simd - 1) / n_simd) * (4 * 118 + 60);
+        const GemvPlan half{n_blocks * 2, 4};
+        if ((n_blocks <= 48 || linear_small_uses_atomics(rows, n_groups, half)) &&
+            (n_blocks <= 48 || cost_half < cost_whole))
+            return half;
+    }
     int max_splits = target_waves / (n_groups > 0 ? n_groups : 1);
     if (max_splits < 1) max_splits = 1;
     if (max_splits > n_blocks) max_splits = n_blocks;
