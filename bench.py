@@ -19,8 +19,9 @@ HIP events around batched graph replays on cold weights; next to the published
 8 TB/s it carries the streaming-read rate and the decode-loop rate measured in
 the same run), ceilings (those two measurements in full), cpu_baseline (the C
 oracle on the host cores), batch_rows (2..128 rows), config1, prefill_gemm
-(M=2048, config 3), moe (config 4), encoder and config5 (K in {2,6,8}, 3INST and
-MCG, 1 and 8 rows; --sweep: K in {2,3,5,6,8} at 1/4/8 rows).
+(M=2048, config 3), moe (config 4), encoder, config5 (K in {2,3,5,6,8} x {3INST,
+MCG} x 1/4/8 rows), eager_ms_per_step (the same steps without a graph) and
+launch_plans (the host-side plan of each of the step's launches).
 """
 
 from __future__ import annotations
@@ -171,8 +172,6 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-extras", action="store_true", help="skip prefill GEMM and MoE figures")
     ap.add_argument("--unfused-qkv", action="store_true", help="run q, k, v as three launches")
-    ap.add_argument("--sweep", action="store_true",
-                    help="also time config 5: the layer at K in {2,3,5,6,8}, 3INST and MCG, 1/4/8 rows")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 64 MiB device-to-device copy (for counter runs: FETCH_SIZE / "
                          "WRITE_SIZE of a transfer of known size)")
@@ -280,6 +279,32 @@ def main():
     event_ms_per_step = float(np.median(event_samples))
     value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
 
+    # the same steps launched eagerly through the module path (ctypes call per launch,
+    # no graph): what EXL3Linear costs a caller that does not capture its decode step
+    eager_samples = []
+    for _ in range(3):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step(i % n_layers)
+        torch.cuda.synchronize()
+        eager_samples.append((time.perf_counter() - t0) * 1e3 / args.steps)
+    eager_ms_per_step = float(np.median(eager_samples))
+
+    # launch plans (box-independent host decisions): a slow box can be told from a bad plan
+    import ctypes
+
+    lib = _lib.load()
+    plans = {}
+    for lin in layers[0]:
+        v = [ctypes.c_int() for _ in range(4)]
+        _lib.check(lib.exl3_linear_plan(1, lin.n_in // 16, lin.n_out // 16, K_BITS, *[ctypes.byref(c) for c in v]),
+                   "exl3_linear_plan")
+        splits, tk, nw, atomic = (c.value for c in v)
+        plans[lin.name] = {"grid": f"{lin.n_out // 128}x{(splits + nw - 1) // nw}", "waves_per_workgroup": nw,
+                           "tile_rows_per_wave": tk, "split": {4: "half block", 8: "one block"}.get(tk, f"{tk // 8} blocks"),
+                           "reduction": "accumulators" if atomic else "partial rows"}
+
     # ---- roofline of the dominant kernel: the one-launch layer kernel (input
     # Hadamard + decode GEMV + split reduction + output Hadamard). The timed step is
     # four launches of it and nothing else, so its average launch duration over the
@@ -339,9 +364,6 @@ def main():
         extras.update(bench_prefill(dev, layers[0], xs))
         extras.update(bench_moe(dev))
         extras.update(bench_encoder(dev))
-        if not args.sweep:
-            extras.update(bench_sweep(dev, layers[0], ks=(2, 6, 8), row_counts=(1, 8)))
-    if args.sweep:
         extras.update(bench_sweep(dev, layers[0]))
 
     out = {
@@ -354,6 +376,7 @@ def main():
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5),
         "ms_per_step_samples": [round(v, 5) for v in samples],
+        "eager_ms_per_step": round(eager_ms_per_step, 5),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -368,6 +391,7 @@ def main():
             "launch": (f"hip-graph replay, {n_layers} layer steps per graph" if graph_all is not None
                        else "eager"),
         },
+        "launch_plans": plans,
         "roofline": roofline,
     }
     out.update(extras)
@@ -571,8 +595,7 @@ def bench_config1(dev):
 
 
 def bench_sweep(dev, layer, ks=(2, 3, 5, 6, 8), row_counts=(1, 4, 8)):
-    """config 5: the config-2 layer at other bit widths and codebooks (the default run
-    takes K in {2, 6, 8} at 1 and 8 rows, --sweep all of K in {2,3,5,6,8} at 1/4/8)."""
+    """config 5: the config-2 layer at K in {2,3,5,6,8} x {3INST, MCG} x 1/4/8 rows."""
     res = {}
     for k in ks:
         total = sum(l.n_in * l.n_out * k // 8 for l in layer)

@@ -265,6 +265,17 @@ int exl3_linear_forward(const uint16_t *x, int rows, const uint16_t *trellis, in
 size_t exl3_linear_workspace_bytes(int rows, int in_features, int out_features, int n_sub);
 
 /*
+ * The launch plan the one-launch layer kernel takes for a shape (rows <=
+ * exl3_gemv_max_rows()), for logs and benchmarks: wave-level splits of the tile rows,
+ * tile rows per split (4 = half a Hadamard block per wave, 8 = one block, 16 = two),
+ * waves per workgroup (4 or 8) and whether the split reduction goes through the 64-bit
+ * accumulators (1) or through partial rows (0). The counterpart of the reference's
+ * split chooser (ponyexl3/mlx/gemv_metal.py:1405-1414). Any output pointer may be NULL.
+ */
+int exl3_linear_plan(int rows, int in_tiles, int out_tiles, int K, int *n_splits,
+                     int *tile_rows_per_split, int *waves_per_workgroup, int *atomic);
+
+/*
  * Error channel of the accumulator reductions (exl3_linear_forward, exl3_moe_forward,
  * exl3_linear_forward_static); no counterpart in the reference, whose kernels have no
  * split state that outlives a launch. The workgroup that finishes a 128-column group

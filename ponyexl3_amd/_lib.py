@@ -64,6 +64,7 @@ PROTOTYPES = {
     ),
     "exl3_linear_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "exl3_counters_status": (_i, [_vp, _sz, _vp]),
+    "exl3_linear_plan": (_i, [_i, _i, _i, _i] + [ctypes.POINTER(_i)] * 4),
     "exl3_linear_static_scratch_bytes": (_sz, []),
     "exl3_linear_static_need_bytes": (_sz, [_i, _i, _i]),
     "exl3_linear_forward_static": (

@@ -659,6 +659,20 @@ EXL3_EXPORT int exl3_gemv_plan(int rows, int in_tiles, int n_groups, int* n_spli
     return EXL3_OK;
 }
 
+EXL3_EXPORT int exl3_linear_plan(int rows, int in_tiles, int out_tiles, int K, int* n_splits,
+                                 int* tile_rows_per_split, int* waves_per_workgroup, int* atomic) {
+    using namespace exl3;
+    if (rows < 1 || rows > kLinearSmallMaxRows || in_tiles < 8 || out_tiles < 8 || in_tiles % 8 ||
+        out_tiles % 8 || K < 1 || K > 8)
+        return EXL3_E_BAD_SHAPE;
+    const GemvPlan plan = plan_linear_small_launch(rows, in_tiles, out_tiles / 8, K);
+    if (n_splits) *n_splits = plan.n_splits;
+    if (tile_rows_per_split) *tile_rows_per_split = plan.tk_per_split;
+    if (waves_per_workgroup) *waves_per_workgroup = plan.wg_waves;
+    if (atomic) *atomic = linear_small_uses_atomics(rows, out_tiles / 8, plan) ? 1 : 0;
+    return EXL3_OK;
+}
+
 EXL3_EXPORT int exl3_gemv_partials(const uint16_t* xh, int rows, int n_sub, const uint16_t* trellis,
                                    int in_tiles, int out_tiles, int K, int cb,
                                    const int32_t* group_sub, const int32_t* group_tile,
