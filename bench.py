@@ -620,9 +620,12 @@ def bench_prefill(dev, layer, xs):
     flop = ms_tot = ms_layer_tot = 0.0
     for lin in layer:
         xh = torch.randn((2048, lin.n_in), generator=g).to(torch.float16).to(dev)
-        ms = _time_ms(lambda: ops.inner_gemm(xh, lin.trellis, K_BITS, CB), reps=10)
-        # the whole layer at 2048 rows: input Hadamard, GEMM, output Hadamard
-        ms_layer = _time_ms(lambda: lin.forward(xh), reps=10)
+        # calls queued back to back (the device never waits for the host between them), as the
+        # layers of a prefill chunk are
+        ms = _time_batch_ms(lambda: ops.inner_gemm(xh, lin.trellis, K_BITS, CB), reps=10, warm=3)
+        # the whole layer at 2048 rows: input rotation, GEMM with the output transform in its
+        # epilogue (split tiles: in the pass that adds their partial tiles)
+        ms_layer = _time_batch_ms(lambda: lin.forward(xh), reps=10, warm=3)
         f = 2.0 * 2048 * lin.n_in * lin.n_out
         per[lin.name] = {"ms": round(ms, 4), "TFLOPs": round(f / ms / 1e9, 1),
                          "layer_ms": round(ms_layer, 4), "layer_TFLOPs": round(f / ms_layer / 1e9, 1)}
@@ -634,14 +637,17 @@ def bench_prefill(dev, layer, xs):
     # context: what a plain fp16 GEMM of the library reaches on this box at the gate+up shape
     a = torch.randn((2048, 5120), generator=g).to(torch.float16).to(dev)
     b = torch.randn((5120, 34816), generator=g).to(torch.float16).to(dev)
-    ms_lib = _time_ms(lambda: torch.matmul(a, b), reps=10)
+    ms_lib = _time_batch_ms(lambda: torch.matmul(a, b), reps=10, warm=3)
     lib_tf = 2.0 * 2048 * 5120 * 34816 / ms_lib / 1e9
     del a, b
     return {"prefill_gemm": {"M": 2048, "TFLOPs": round(tf, 1), "peak": MFMA_F16_PEAK_TFLOPS,
                              "layer_TFLOPs_with_hadamards": round(flop / ms_layer_tot / 1e9, 1),
                              "library_fp16_gemm_TFLOPs_gate_up_shape": round(lib_tf, 1),
-                             "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "bound": "mfma",
-                             "kernel": "gemm_kernel<K=4, cb=3INST>", "per_linear": per}}
+                             "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                             "layer_frac": round(flop / ms_layer_tot / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
+                             "bound": "mfma", "kernel": "gemm_kernel<K=4, cb=3INST>",
+                             "timing": "HIP events around ten calls queued back to back",
+                             "per_linear": per}}
 
 
 def bench_encoder(dev):

@@ -102,7 +102,8 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
     float* __restrict__ partial, int rows_arg, size_t ldx, size_t ldy, int in_tiles, int out_tiles,
     int tn_offset_arg, int tn_count_arg, int n_row_blocks, int full_tiles, int split,
     int ksteps_per_split, const int4* __restrict__ group_tab, int group_tiles, int n_groups,
-    const int* __restrict__ block_sub, size_t sub_stride) {
+    const int* __restrict__ block_sub, size_t sub_stride, const half_t* __restrict__ post_svh,
+    const half_t* __restrict__ post_bias, half_t* __restrict__ post_out, size_t ldo) {
     extern __shared__ __attribute__((aligned(16))) half_t smem[];
     constexpr int BM = 32 * MI;
     constexpr int STAGE_A = BM * 64, STAGE_B = kGemmStageB;
@@ -328,6 +329,93 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
 
     // acc[i][j] is D^T: lane holds columns 4*(lane/16)+0..3 of row lane%16
     const int col0 = g * kGemmBN + wn * 64 + (lane >> 4) * 4;
+    if (post_out && work.partial_unit < 0) {
+        // Output transform of a whole tile inside the kernel (ponyexl3/ref/forward.py:41-45):
+        // y16 = fp16(acc) goes to LDS, then Z = Y16 x H128 per 128-column block runs on the
+        // matrix pipe as well - 128 more MFMAs per wave next to the 64 of every k-step, instead
+        // of a pass that reads and writes all of y again. H is symmetric with entries +-1,
+        // exact in fp16, so the products are exact and the sums are fp32 as in the butterfly
+        // form (another order of additions: the fp16 result can differ from the separate pass
+        // in its last bit). The fragments of H come from four register sets per lane: entry
+        // (k, n) has sign parity(k & n); with n = 16 nt + fr and k = 32 ks + 8 q + t the parity
+        // splits into a part the lane knows (fr, q, t), a part that needs nt & 1 and a part
+        // that is the same for every lane of the instruction (nt >> 1 and ks, compile time).
+        constexpr int kYLd = kGemmBN + 8;  // row stride in halfs: 16-byte reads of 16 rows hit 64 banks
+        half_t* ys = smem;
+        const int q = lane >> 4;
+#pragma unroll
+        for (int ii = 0; ii < MI; ii++) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                half4_t o;
+                o.x = (half_t)acc[ii][j].x;
+                o.y = (half_t)acc[ii][j].y;
+                o.z = (half_t)acc[ii][j].z;
+                o.w = (half_t)acc[ii][j].w;
+                *reinterpret_cast<half4_t*>(ys + (wm * (16 * MI) + ii * 16 + fr) * kYLd + wn * 64 +
+                                            j * 16 + q * 4) = o;
+            }
+        }
+        uint32_t hsign[2][2][4];  // [nt & 1][uniform flip][pair of k-slots]
+        {
+            const uint32_t lane_flip0 = ((fr >> 3) & q & 1) ? 0x80008000u : 0u;
+            const uint32_t lane_flip1 = lane_flip0 ^ ((q >> 1) ? 0x80008000u : 0u);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t lo = __builtin_popcount(fr & 7 & (2 * i)) & 1;
+                const uint32_t hi = __builtin_popcount(fr & 7 & (2 * i + 1)) & 1;
+                const uint32_t base = 0x3C003C00u | (lo << 15) | (hi << 31);
+                hsign[0][0][i] = base ^ lane_flip0;
+                hsign[0][1][i] = base ^ lane_flip0 ^ 0x80008000u;
+                hsign[1][0][i] = base ^ lane_flip1;
+                hsign[1][1][i] = base ^ lane_flip1 ^ 0x80008000u;
+            }
+        }
+        __syncthreads();
+        constexpr int U = MI / 2;  // (16-row tile, 128-column block) units per wave
+        static_for<0, U>([&](auto ui) {
+            const int u = wave * U + ui.value;
+            const int rt = u >> 1, blk = u & 1;
+            float4_t z[8];
+#pragma unroll
+            for (int nt = 0; nt < 8; nt++) z[nt] = float4_t{0.f, 0.f, 0.f, 0.f};
+            const half_t* yrow = ys + (rt * 16 + fr) * kYLd + blk * 128 + q * 8;
+            static_for<0, 4>([&](auto ks) {
+                const half8_t yf = *reinterpret_cast<const half8_t*>(yrow + ks.value * 32);
+                static_for<0, 8>([&](auto nt) {
+                    constexpr int uni = ((nt.value >> 1) & ks.value & 1) ^
+                                        ((nt.value >> 2) & (ks.value >> 1) & 1);
+                    const uint4_t hv = {hsign[nt.value & 1][uni][0], hsign[nt.value & 1][uni][1],
+                                        hsign[nt.value & 1][uni][2], hsign[nt.value & 1][uni][3]};
+                    z[nt.value] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                        __builtin_bit_cast(half8_t, hv), yf, z[nt.value], 0, 0, 0);
+                });
+            });
+            const int r = m0 + rt * 16 + fr;
+            const int cb0 = g * kGemmBN + blk * 128 + q * 4;
+            if (r < rows && cb0 < tn_count * 16) {  // (a half-width last block has no second block)
+#pragma unroll
+                for (int nt = 0; nt < 8; nt++) {
+                    const int col = cb0 + nt * 16;
+                    float v[4] = {z[nt].x, z[nt].y, z[nt].z, z[nt].w};
+                    half4_t sv, bv;
+                    if (post_svh) sv = *reinterpret_cast<const half4_t*>(post_svh + col);
+                    if (post_bias) bv = *reinterpret_cast<const half4_t*>(post_bias + col);
+                    half4_t o;
+#pragma unroll
+                    for (int c = 0; c < 4; c++) {
+                        float a = __fmul_rn(v[c], 0.088388347648318440550f);  // 1/sqrt(128)
+                        if (post_svh) a = __fmul_rn(a, (float)sv[c]);
+                        half_t h = (half_t)a;
+                        if (post_bias) h = h + bv[c];
+                        o[c] = h;
+                    }
+                    *reinterpret_cast<half4_t*>(post_out + (size_t)r * ldo + col) = o;
+                }
+            }
+        });
+        return;
+    }
     if (g * kGemmBN + wn * 64 >= tn_count * 16) return;  // upper half of a half-width last block
     if (work.partial_unit < 0) {
 #pragma unroll
@@ -401,12 +489,12 @@ __global__ __launch_bounds__(256) void gemm_fixup_kernel(const float* __restrict
 // cast, bias.
 template <int MI>
 __global__ __launch_bounds__(256) void gemm_fixup_post_kernel(
-    const float* __restrict__ partial, int rows, int tn_count, int n_row_blocks, int split,
-    const half_t* __restrict__ svh, const half_t* __restrict__ bias, half_t* __restrict__ out,
-    size_t ldo) {
+    const float* __restrict__ partial, int rows, int tn_count, int n_row_blocks, int full_tiles,
+    int split, const half_t* __restrict__ svh, const half_t* __restrict__ bias,
+    half_t* __restrict__ out, size_t ldo) {
     constexpr int BM = 32 * MI;
     constexpr float kScale = 0.088388347648318440550f;  // 1/sqrt(128)
-    const int tile = blockIdx.x;
+    const int tile = full_tiles + blockIdx.x;
     const int g = tile / n_row_blocks;
     const int m0 = (tile % n_row_blocks) * BM;
     const int lane = threadIdx.x & 63;
@@ -530,7 +618,10 @@ static int launch_gemm_mi(const GemmPlan& p, const uint16_t* xh, int rows, size_
                           int tn_count, uint16_t* y_out, size_t ldy, float* partial,
                           hipStream_t stream, const GemmPost* post, const int32_t* block_sub,
                           size_t sub_stride) {
-    constexpr size_t lds = (2 * (size_t)(32 * MI) * 64 + 2 * (size_t)kGemmStageB) * sizeof(half_t);
+    // two stages of A and B, or (output transform inside the kernel) the fp16 tile with padded rows
+    constexpr size_t lds_stages = (2 * (size_t)(32 * MI) * 64 + 2 * (size_t)kGemmStageB) * sizeof(half_t);
+    constexpr size_t lds_tile = (size_t)(32 * MI) * (kGemmBN + 8) * sizeof(half_t);
+    constexpr size_t lds = lds_stages > lds_tile ? lds_stages : lds_tile;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_kernel<K, CB, MI>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
         return EXL3_E_LAUNCH;
@@ -539,14 +630,23 @@ static int launch_gemm_mi(const GemmPlan& p, const uint16_t* xh, int rows, size_
         reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<const half_t*>(xh),
         reinterpret_cast<half_t*>(y_out), partial, rows, ldx, ldy, in_tiles, out_tiles, tn_offset,
         tn_count, p.n_row_blocks, p.full_tiles, p.split, p.ksteps_per_split, nullptr, 0, 0,
-        block_sub, sub_stride);
+        block_sub, sub_stride, post ? reinterpret_cast<const half_t*>(post->svh) : nullptr,
+        post ? reinterpret_cast<const half_t*>(post->bias) : nullptr,
+        post ? reinterpret_cast<half_t*>(post->out) : nullptr, post ? post->ldo : 0);
     if (int rc = launch_status()) return rc;
-    if (post) {  // only passed when every tile is split
-        gemm_fixup_post_kernel<MI><<<dim3((unsigned)p.split_tiles, 4 * MI), dim3(256), 0, stream>>>(
-            partial, rows, tn_count, p.n_row_blocks, p.split,
-            reinterpret_cast<const half_t*>(post->svh), reinterpret_cast<const half_t*>(post->bias),
-            reinterpret_cast<half_t*>(post->out), post->ldo);
-        return launch_status();
+    if (post) {
+        // whole tiles were transformed by the kernel itself; split tiles by the pass that
+        // adds their partial tiles
+        if (p.split_tiles > 0) {
+            gemm_fixup_post_kernel<MI>
+                <<<dim3((unsigned)p.split_tiles, 4 * MI), dim3(256), 0, stream>>>(
+                    partial, rows, tn_count, p.n_row_blocks, p.full_tiles, p.split,
+                    reinterpret_cast<const half_t*>(post->svh),
+                    reinterpret_cast<const half_t*>(post->bias),
+                    reinterpret_cast<half_t*>(post->out), post->ldo);
+            return launch_status();
+        }
+        return EXL3_OK;
     }
     if (p.split_tiles > 0) {
         gemm_fixup_kernel<MI><<<dim3((unsigned)p.split_tiles, 4 * MI), dim3(256), 0, stream>>>(
@@ -579,10 +679,13 @@ int launch_gemm(const uint16_t* xh, int rows, size_t ldx, const uint16_t* trelli
     if ((long long)p.full_tiles + (long long)p.split_tiles * p.split > 0x7fffffffLL)
         return EXL3_E_BAD_SHAPE;
     float* partial = reinterpret_cast<float*>(workspace);
-    // the output transform rides on the fix-up when there is nothing but split tiles
-    const bool fold = post && post->out && post_done && p.split > 1 && p.full_tiles == 0 &&
-                      tn_offset == 0 && post->ldo >= (size_t)tn_count * 16 && post->ldo % 4 == 0 &&
-                      !(reinterpret_cast<uintptr_t>(post->out) & 7);
+    // the output transform rides on the kernel's epilogue (whole tiles) and on the fix-up
+    // (split tiles); it needs whole Hadamard blocks of the whole width
+    const bool fold = post && post->out && post_done && tn_offset == 0 && tn_count % 8 == 0 &&
+                      post->ldo >= (size_t)tn_count * 16 && post->ldo % 4 == 0 &&
+                      !(reinterpret_cast<uintptr_t>(post->out) & 7) &&
+                      !(reinterpret_cast<uintptr_t>(post->svh) & 7) &&
+                      !(reinterpret_cast<uintptr_t>(post->bias) & 7);
     const GemmPost* fp = fold ? post : nullptr;
     const int rc = dispatch_k_cb(K, cb, [&](auto k, auto c) {
         if (p.mi == 2)
@@ -617,7 +720,7 @@ static int launch_gemm_grouped_mi(const uint16_t* xh, int n_rows, size_t ldx,
         reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<const half_t*>(xh),
         reinterpret_cast<half_t*>(y_out), nullptr, n_rows, ldx, ldy, in_tiles, out_tiles, tn_base,
         group_tiles, 1, 0, 1, in_tiles / 4, reinterpret_cast<const int4*>(group_tab), group_tiles,
-        n_groups, nullptr, 0);
+        n_groups, nullptr, 0, nullptr, nullptr, nullptr, 0);
     return launch_status();
 }
 

@@ -88,34 +88,55 @@ __global__ __launch_bounds__(256) void had_pre_wide_kernel(const half_t* __restr
                                                            half_t* __restrict__ xh, int n,
                                                            int n_sub, RowMap map) {
     const int lane = threadIdx.x & 63;
-    const size_t rs = blockIdx.x;
-    if (!map.row_ok(rs, suh != nullptr)) return;
-    // source row and scale vector: (row, sub) product for stacked siblings, or
-    // per-row tables for rows that were sorted by expert
-    const half_t* xr = x + (map.per_row ? map.in_row(rs) : rs / n_sub) * (size_t)n;
-    const half_t* sr =
-        suh ? suh + (map.per_row ? map.scale_row(rs) * map.scale_ld : (rs % n_sub) * (size_t)n)
-            : nullptr;
-    half_t* orow = xh + map.out_row(rs) * (size_t)n;
-    for (int c = (blockIdx.y * 256 + threadIdx.x) * 8; c < n; c += 2048 * gridDim.y) {
-        float v[8], sv[8];
-        halfs_to_floats(*reinterpret_cast<const uint4_t*>(xr + c), v);
-        if (sr) {
-            halfs_to_floats(*reinterpret_cast<const uint4_t*>(sr + c), sv);
+    // One workgroup per source row: per-row tables (rows sorted by expert) give its
+    // source, scale vector and destination; otherwise the row is rotated once per stacked
+    // sibling (scale vector s, destination row r * n_sub + s) from a single read.
+    const size_t r = blockIdx.x;
+    if (!map.row_ok(r, suh != nullptr)) return;
+    const half_t* xr = x + (map.per_row ? map.in_row(r) : r) * (size_t)n;
+    const int subs = map.per_row ? 1 : n_sub;
+    // up to four 16-byte chunks of the row in flight per lane
+    const int c0 = (blockIdx.y * 256 + threadIdx.x) * 8, cstep = 2048 * gridDim.y;
+    for (int cb = c0; cb < n; cb += 4 * cstep) {
+        uint4_t raw[4];
 #pragma unroll
-            for (int j = 0; j < 8; j++) v[j] = v[j] * sv[j];
-        }
-        wht128_wide(v, lane);
-        uint4_t o;
-        uint32_t* ow = reinterpret_cast<uint32_t*>(&o);
+        for (int i = 0; i < 4; i++)
+            if (cb + i * cstep < n) raw[i] = *reinterpret_cast<const uint4_t*>(xr + cb + i * cstep);
+        for (int s = 0; s < subs; s++) {
+            const half_t* sr =
+                suh ? suh + (map.per_row ? map.scale_row(r) * map.scale_ld : s * (size_t)n) : nullptr;
+            half_t* orow = xh + (map.per_row ? map.out_row(r) : r * n_sub + s) * (size_t)n;
+            uint4_t sraw[4];
+            if (sr) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            half2_t h;
-            h.x = (half_t)(v[2 * i] * kHadScale);
-            h.y = (half_t)(v[2 * i + 1] * kHadScale);
-            ow[i] = half2_to_bits(h);
+                for (int i = 0; i < 4; i++)
+                    if (cb + i * cstep < n)
+                        sraw[i] = *reinterpret_cast<const uint4_t*>(sr + cb + i * cstep);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int c = cb + i * cstep;
+                if (c >= n) break;
+                float v[8], sv[8];
+                halfs_to_floats(raw[i], v);
+                if (sr) {
+                    halfs_to_floats(sraw[i], sv);
+#pragma unroll
+                    for (int j = 0; j < 8; j++) v[j] = v[j] * sv[j];
+                }
+                wht128_wide(v, lane);
+                uint4_t o;
+                uint32_t* ow = reinterpret_cast<uint32_t*>(&o);
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    half2_t h;
+                    h.x = (half_t)(v[2 * k] * kHadScale);
+                    h.y = (half_t)(v[2 * k + 1] * kHadScale);
+                    ow[k] = half2_to_bits(h);
+                }
+                *reinterpret_cast<uint4_t*>(orow + c) = o;
+            }
         }
-        *reinterpret_cast<uint4_t*>(orow + c) = o;
     }
 }
 
@@ -129,34 +150,45 @@ __global__ __launch_bounds__(256) void had_post_wide_kernel(const half_t* __rest
     if (svh && map.per_row) svh += map.scale_row(rs) * map.scale_ld;
     const half_t* yr = y + map.in_row(rs) * (size_t)n;
     half_t* orow = out + map.out_row(rs) * (size_t)n;
-    for (int c = (blockIdx.y * 256 + threadIdx.x) * 8; c < n; c += 2048 * gridDim.y) {
-        float v[8], sv[8];
-        halfs_to_floats(*reinterpret_cast<const uint4_t*>(yr + c), v);
-        wht128_wide(v, lane);
-        if (svh) halfs_to_floats(*reinterpret_cast<const uint4_t*>(svh + c), sv);
-        uint4_t bq = {0u, 0u, 0u, 0u};
-        if (bias) bq = *reinterpret_cast<const uint4_t*>(bias + c);
-        const uint32_t* bw = reinterpret_cast<const uint32_t*>(&bq);
-        uint4_t o;
-        uint32_t* ow = reinterpret_cast<uint32_t*>(&o);
+    // up to four 16-byte chunks of the row in flight per lane
+    const int c0 = (blockIdx.y * 256 + threadIdx.x) * 8, cstep = 2048 * gridDim.y;
+    for (int cb = c0; cb < n; cb += 4 * cstep) {
+        uint4_t raw[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (cb + i * cstep < n) raw[i] = *reinterpret_cast<const uint4_t*>(yr + cb + i * cstep);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            float a = v[2 * i] * kHadScale, b = v[2 * i + 1] * kHadScale;
-            if (svh) {
-                a = a * sv[2 * i];
-                b = b * sv[2 * i + 1];
+            const int c = cb + i * cstep;
+            if (c >= n) break;
+            float v[8], sv[8];
+            halfs_to_floats(raw[i], v);
+            wht128_wide(v, lane);
+            if (svh) halfs_to_floats(*reinterpret_cast<const uint4_t*>(svh + c), sv);
+            uint4_t bq = {0u, 0u, 0u, 0u};
+            if (bias) bq = *reinterpret_cast<const uint4_t*>(bias + c);
+            const uint32_t* bw = reinterpret_cast<const uint32_t*>(&bq);
+            uint4_t o;
+            uint32_t* ow = reinterpret_cast<uint32_t*>(&o);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                float a = v[2 * k] * kHadScale, b = v[2 * k + 1] * kHadScale;
+                if (svh) {
+                    a = a * sv[2 * k];
+                    b = b * sv[2 * k + 1];
+                }
+                half2_t h;
+                h.x = (half_t)a;
+                h.y = (half_t)b;
+                if (bias) {
+                    const half2_t bv = bits_to_half2(bw[k]);
+                    h.x = h.x + bv.x;
+                    h.y = h.y + bv.y;
+                }
+                ow[k] = half2_to_bits(h);
             }
-            half2_t h;
-            h.x = (half_t)a;
-            h.y = (half_t)b;
-            if (bias) {
-                const half2_t bv = bits_to_half2(bw[i]);
-                h.x = h.x + bv.x;
-                h.y = h.y + bv.y;
-            }
-            ow[i] = half2_to_bits(h);
+            *reinterpret_cast<uint4_t*>(orow + c) = o;
         }
-        *reinterpret_cast<uint4_t*>(orow + c) = o;
     }
 }
 
@@ -276,7 +308,7 @@ int launch_had_pre(const uint16_t* x, int rows, int n, const uint16_t* suh, int 
     if (grid > 0x7FFFFFFFLL) return EXL3_E_BAD_SHAPE;
     if ((long long)rows * n_sub >= kWideMinRows && aligned16(x) && aligned16(xh) &&
         (!suh || aligned16(suh))) {
-        had_pre_wide_kernel<<<dim3((unsigned)(rows * n_sub), wide_row_parts((long long)rows * n_sub, n)),
+        had_pre_wide_kernel<<<dim3((unsigned)rows, wide_row_parts((long long)rows, n)),
                               dim3(256), 0, stream>>>(
             reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(suh),
             reinterpret_cast<half_t*>(xh), n, n_sub, RowMap{});

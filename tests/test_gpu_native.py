@@ -32,12 +32,18 @@ def test_public_weight_matches_oracle(cuda, oracle, k, mcg, mul1, n_in, n_out):
 
 
 def test_public_weight_equals_identity_through_the_module(cuda):
-    """The fold is by construction the exact module applied to the identity."""
+    """The fold is the module applied to the identity. Both round the same fp32 sums to
+    fp16; the module's prefill path adds the 128 terms of the output Hadamard on the
+    matrix pipe, the fold in butterfly order, so a result that sits on a rounding boundary
+    can come out one fp16 step apart."""
     from ponyexl3_amd import EXL3Linear, make_exl3_layer, native
 
     layer = make_exl3_layer(k=4, in_features=256, out_features=256, seed=9)
     eye = torch.eye(256, dtype=torch.float16, device=cuda)
-    assert torch.equal(native.public_weight(layer, device=cuda), EXL3Linear(layer)(eye))
+    fold, module = native.public_weight(layer, device=cuda).float(), EXL3Linear(layer)(eye).float()
+    step = torch.maximum(fold.abs(), module.abs()) * 2.0 ** -10 + 2.0 ** -24  # one fp16 step at that size
+    assert bool(((fold - module).abs() <= step).all())
+    assert float((fold != module).float().mean()) < 0.01
 
 
 @pytest.mark.parametrize("bias", [False, True])
