@@ -94,7 +94,7 @@ EXL3_EXPORT int exl3_linear_forward(const uint16_t* x, int rows, const uint16_t*
         const int n_groups = out_tiles / 8;
         const GemvPlan plan = plan_gemv(rows, in_tiles, n_groups);
         float* partial = reinterpret_cast<float*>(second);
-        if (counters) {
+        if (counters && !exact_weights()) {
             // one launch: rotation, GEMV, split reduction and output transform fused;
             // the counters array holds the 64-bit accumulators (two ints each)
             const size_t need = linear_small_counter_ints(rows, out_features);
@@ -292,6 +292,7 @@ EXL3_EXPORT int exl3_linear_forward_static(const uint16_t* x, int rows, const ui
     if (rows < 1 || in_tiles < 8 || out_tiles < 8 || in_tiles % 8 || out_tiles % 8 || n_sub < 1)
         return EXL3_E_BAD_SHAPE;
     if (rows > kLinearSmallMaxRows) return EXL3_E_UNSUPPORTED;  // only the one-launch kernel
+    if (exact_weights()) return EXL3_E_UNSUPPORTED;  // the chain that rounds the weights needs a workspace
     if (n_sub > 1 && (!group_sub || !suh)) return EXL3_E_BAD_INDEX;
     const int n_groups = out_tiles / 8;
     const GemvPlan plan = plan_linear_small_launch(rows, in_tiles, n_groups, K);

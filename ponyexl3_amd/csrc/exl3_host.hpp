@@ -171,6 +171,16 @@ inline int env_int(const char* name, int dflt, int lo, int hi) {
     return x < lo ? lo : (x > hi ? hi : x);
 }
 
+// EXL3_EXACT_WEIGHTS=1: every product uses the weight rounded to fp16, as the reference
+// defines it. The one-launch layer kernel and the down projection of the MoE chain
+// multiply by the exact sum of the weight's two fp16 halves instead (one VALU instruction
+// less per weight; 4-5e-4 rel-L2 on a layer's output, against 5-7e-5); with the knob set
+// the entry points take their multi-launch chains, whose kernels round first.
+inline bool exact_weights() {
+    static const int v = env_int("EXL3_EXACT_WEIGHTS", 0, 0, 1);
+    return v != 0;
+}
+
 // Polls a finishing workgroup spends on accumulators whose counts are not complete yet
 // before it gives up (EXL3_SPIN_LIMIT; read at every launch so that a test can lower it).
 inline int reduction_spin_limit() { return env_int("EXL3_SPIN_LIMIT", 1 << 22, 1, 1 << 30); }

@@ -26,7 +26,9 @@ struct XChunk {
     uint4_t v[(MT + 3) / 4];
 };
 
-template <int MT>
+// EXACT (weights rounded to fp16 before the product, see dot_tile_row_exact): the block is
+// staged once per value and chunk c = input rows 8c..8c+7 of the tile row.
+template <int MT, bool EXACT = false>
 __device__ __forceinline__ XChunk<MT> load_x_chunk(half_t (*xw)[kXwLd], int row_in_block, int xlane,
                                                    int c) {
     constexpr int NQ = (MT + 3) / 4;
@@ -35,7 +37,8 @@ __device__ __forceinline__ XChunk<MT> load_x_chunk(half_t (*xw)[kXwLd], int row_
     for (int q = 0; q < NQ; q++) {
         int m = 4 * q + xlane;
         if (m > MT - 1) m = MT - 1;  // rows past the batch repeat a staged row; never used
-        t.v[q] = *reinterpret_cast<const uint4_t*>(&xw[m][row_in_block * 32 + 8 * c]);
+        t.v[q] = *reinterpret_cast<const uint4_t*>(
+            &xw[m][EXACT ? row_in_block * 16 + 8 * c : row_in_block * 32 + 8 * c]);
     }
     return t;
 }
@@ -93,6 +96,39 @@ __device__ __forceinline__ void dot_tile_row(const LaneWords<K>& lw, LoadChunk&&
     issue(std::integral_constant<int, 15>{});
 }
 
+// The same with the weights as the reference defines them, rounded to fp16 (the half add
+// of ponyexl3/ref/codebook.py:45-51) before they are multiplied: four weights per matrix
+// instruction against four activations. 32 more VALU instructions per tile row than the
+// unsummed form, whose products carry the exact sum of the two halves instead - a relative
+// difference of up to 2^-11 per weight, 4-5e-4 rel-L2 on a layer's output. Chains of
+// layers with a nonlinearity in between (the MoE experts) take this form for the
+// projections in front of it.
+template <int K, int CB, int MT, class LoadChunk>
+__device__ __forceinline__ void dot_tile_row_exact(const LaneWords<K>& lw, LoadChunk&& load_chunk,
+                                                   float4_t (&accv)[2][(MT + 3) / 4]) {
+    constexpr int NQ = (MT + 3) / 4;
+    const XChunk<MT> xc[2] = {load_chunk(0), load_chunk(1)};
+    half2_t wp[16];
+    decode_lane<K, CB>(lw, wp);
+    // fresh-row groups outermost: consecutive MFMAs then write different accumulators
+#pragma unroll
+    for (int j4 = 0; j4 < 4; j4++) {  // input rows 4*j4 .. 4*j4+3 of the tile
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            const uint4_t xv = xc[j4 >> 1].v[q];
+            const uint2_t xa = (j4 & 1) ? uint2_t{xv.z, xv.w} : uint2_t{xv.x, xv.y};
+#pragma unroll
+            for (int cs = 0; cs < 2; cs++) {
+                const uint2_t wb = {half2_to_bits(wp[8 * cs + 2 * j4]),
+                                    half2_to_bits(wp[8 * cs + 2 * j4 + 1])};
+                accv[cs][q] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4_t, xa),
+                                                               __builtin_bit_cast(half4_t, wb),
+                                                               accv[cs][q], 0, 0, 0);
+            }
+        }
+    }
+}
+
 template <int K>
 __device__ __forceinline__ void load_lane_words_nt(const uint32_t* __restrict__ p,
                                                    uint32_t (&own)[K]) {
@@ -143,7 +179,8 @@ __device__ __forceinline__ void issue_first_rows(Words base, size_t row_words, i
     }
 }
 
-template <int K, int CB, int MT, bool ROTATE, bool HALF, bool GUARD, bool PRELOADED>
+template <int K, int CB, int MT, bool ROTATE, bool HALF, bool GUARD, bool PRELOADED,
+          bool EXACT = false>
 __device__ __forceinline__ void stream_block_rows_at(const uint32_t* __restrict__ base,
                                                      size_t row_words, int tk_begin, int tk_end,
                                                      const half_t* const (&xrow)[MT], int rows,
@@ -176,8 +213,13 @@ __device__ __forceinline__ void stream_block_rows_at(const uint32_t* __restrict_
                 o.x = (half_t)__fmul_rn(a, kHadScaleF);
                 o.y = (half_t)__fmul_rn(b, kHadScaleF);
             }
-            const uint32_t lo = half_to_bits(o.x), hi = half_to_bits(o.y);
-            *reinterpret_cast<uint2_t*>(&xw[m][4 * lane]) = uint2_t{lo | (lo << 16), hi | (hi << 16)};
+            if constexpr (EXACT) {
+                *reinterpret_cast<half2_t*>(&xw[m][2 * lane]) = o;
+            } else {
+                const uint32_t lo = half_to_bits(o.x), hi = half_to_bits(o.y);
+                *reinterpret_cast<uint2_t*>(&xw[m][4 * lane]) =
+                    uint2_t{lo | (lo << 16), hi | (hi << 16)};
+            }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -190,9 +232,11 @@ __device__ __forceinline__ void stream_block_rows_at(const uint32_t* __restrict_
         for (int q = 0; q < NQ; q++) accv[cs][q] = float4_t{0.f, 0.f, 0.f, 0.f};
     const int xlane = lane & 3;
     auto consume = [&](const uint32_t (&words)[K], uint32_t prev, int row_in_block) {
-        dot_tile_row<K, CB, MT>(
-            make_lane_words<K>(prev, words),
-            [&](int c) { return load_x_chunk<MT>(xw, row_in_block, xlane, c); }, accv);
+        auto chunk = [&](int c) { return load_x_chunk<MT, EXACT>(xw, row_in_block, xlane, c); };
+        if constexpr (EXACT)
+            dot_tile_row_exact<K, CB, MT>(make_lane_words<K>(prev, words), chunk, accv);
+        else
+            dot_tile_row<K, CB, MT>(make_lane_words<K>(prev, words), chunk, accv);
     };
     auto add_up = [&]() {
 #pragma unroll
@@ -252,7 +296,7 @@ __device__ __forceinline__ void stream_block_rows_at(const uint32_t* __restrict_
 }
 
 // The same over `rows` consecutive rows of a row-major activation matrix.
-template <int K, int CB, int MT, bool ROTATE, bool HALF = false>
+template <int K, int CB, int MT, bool ROTATE, bool HALF = false, bool EXACT = false>
 __device__ __forceinline__ void stream_block_rows(const uint32_t* __restrict__ base,
                                                   size_t row_words, int tk_begin, int tk_end,
                                                   const half_t* __restrict__ x, size_t x_stride,
@@ -263,7 +307,7 @@ __device__ __forceinline__ void stream_block_rows(const uint32_t* __restrict__ b
 #pragma unroll
     for (int m = 0; m < MT; m++) xrow[m] = x + (size_t)(m < rows ? m : 0) * x_stride;
     uint32_t buf[kStreamSlots][K];
-    stream_block_rows_at<K, CB, MT, ROTATE, HALF, false, false>(
+    stream_block_rows_at<K, CB, MT, ROTATE, HALF, false, false, EXACT>(
         base, row_words, tk_begin, tk_end, xrow, rows, suh_row, xw, lane, acc, buf);
 }
 

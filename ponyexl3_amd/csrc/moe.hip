@@ -262,7 +262,7 @@ __global__ __launch_bounds__(NW * 64) void moe_gateup_kernel(
         const size_t row_words = (size_t)E * 2 * (H >> 4) * (8 * K);
         const uint32_t* base =
             gu_trellis + ((size_t)(p * E + e) * (H >> 4) + 8 * hg) * (8 * K) + lane * K;
-        stream_block_rows<K, CB, 1, true, kHalf>(base, row_words, tk0, tk0 + (kHalf ? 4 : 8),
+        stream_block_rows<K, CB, 1, true, kHalf, true>(base, row_words, tk0, tk0 + (kHalf ? 4 : 8),
                                                  x + (size_t)(s / top_k) * D, (size_t)D, 1,
                                                  gu_suh + ((size_t)e * 2 + p) * D, xs[wave], lane,
                                                  acc);
@@ -340,7 +340,7 @@ __global__ __launch_bounds__(512) void moe_gateup_pair_kernel(
         const size_t row_words = (size_t)E * 2 * (H >> 4) * (8 * K);
         const uint32_t* base =
             gu_trellis + ((size_t)(p * E + e) * (H >> 4) + 8 * hg) * (8 * K) + lane * K;
-        stream_block_rows<K, CB, 1, true, HALF>(base, row_words, tk0, tk0 + (HALF ? 4 : 8),
+        stream_block_rows<K, CB, 1, true, HALF, true>(base, row_words, tk0, tk0 + (HALF ? 4 : 8),
                                                 x + (size_t)(s / top_k) * D, (size_t)D, 1,
                                                 gu_suh + ((size_t)e * 2 + p) * D, xs[wave], lane,
                                                 acc);
@@ -627,7 +627,7 @@ __global__ __launch_bounds__(NW * 64) void moe_gateup_grouped_kernel(
         const half_t* xrow[kGroupRows];
 #pragma unroll
         for (int m = 0; m < kGroupRows; m++) xrow[m] = x + (size_t)(group_slot(grp, m) / top_k) * D;
-        stream_block_rows_at<K, CB, kGroupRows, true, kHalf, true, true>(
+        stream_block_rows_at<K, CB, kGroupRows, true, kHalf, true, true, true>(
             base, row_words, tk0, tk1, xrow, grp.n, gu_suh + ((size_t)e * 2 + p) * D, xs[wave],
             lane, acc, buf);
     }
@@ -985,7 +985,7 @@ EXL3_EXPORT int exl3_moe_forward(const uint16_t* x, int tokens, const int32_t* i
     float* part_dn = reinterpret_cast<float*>(base + w.o_part_dn);
     const int slots = tokens * top_k;
 
-    if (counters) {
+    if (counters && !exact_weights()) {
         // two launches: gate/up + GLU + rotation, then down
         const int hblocks = H / 128, dblocks = D / 128;
         if (counters_len < (size_t)slots * (hblocks + dblocks)) return EXL3_E_WORKSPACE;
