@@ -45,7 +45,7 @@ CB = 0
 # rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE), each scaled
 # by what the same counter reads for a plain copy of known size; see
 # profiles/linear_small_k4_config2_pmc.txt.
-TRAFFIC_BYTES_PER_STEP = 201_456_400
+TRAFFIC_BYTES_PER_STEP = 200_702_566
 
 # (name, in, [member out sizes]) of the config-2 layer; several members = sibling-fused
 LAYER_FUSED_QKV = [
@@ -337,6 +337,7 @@ def main():
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
         "traffic": TRAFFIC_BYTES_PER_STEP,
+        "traffic_per_launch": TRAFFIC_BYTES_PER_STEP // 4,
         "traffic_source": "profiles/linear_small_k4_config2_pmc.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this "
                           "script, scaled by a 64 MiB copy); a constant, not measured in this run",
         "bytes_per_launch": "in*out*K/8 of the launch's linear(s): 45.2 MB on average over the four launches of a "
@@ -474,7 +475,7 @@ def bench_ceilings(dev):
     """What this GPU delivers, measured in the same run: a streaming read of cold
     memory (the denominator next to the published 8 TB/s), and the small-batch
     kernels' inner loop on its own (wave-wide load, per-lane decode of 32 codewords,
-    8 matrix-pipe dot products; one workgroup of 16 waves per CU, 128 tile rows per
+    16 matrix-pipe dot products; one workgroup of 16 waves per CU, 128 tile rows per
     wave, no Hadamard, no reduction): the rate the VALU instruction sequence of the
     bit-exact decode allows before any layer structure is added. 'cold' walks over a
     2 GiB buffer so that every launch reads memory no earlier launch of the
@@ -486,6 +487,7 @@ def bench_ceilings(dev):
     from ponyexl3_amd import _lib
 
     lib = _lib.load_diag()
+    main_lib = _lib.load()
     total = 2 << 30
     buf = torch.randint(-2**31, 2**31 - 1, (total // 4,), dtype=torch.int32, device=dev)
     out = torch.zeros(4096 * 1024, dtype=torch.float32, device=dev)
@@ -555,8 +557,14 @@ def bench_ceilings(dev):
     # wave's first four tile rows arriving from cold memory.
     phases = {}
     n_rows = total // (256 * K_BITS)
-    for name, gx, gy, threads in (("qkv_proj", 80, 20, 256), ("o_proj", 40, 16, 256),
-                                  ("gate_up", 272, 5, 512), ("down_proj", 40, 34, 256)):
+    grids = []
+    for name, n_in, outs in LAYER:  # the grids the host plans for these launches
+        v = [ctypes.c_int() for _ in range(4)]
+        _lib.check(main_lib.exl3_linear_plan(1, n_in // 16, sum(outs) // 16, K_BITS, *[ctypes.byref(c) for c in v]),
+                   "exl3_linear_plan")
+        splits, _, nw, _ = (c.value for c in v)
+        grids.append((name, sum(outs) // 128, (splits + nw - 1) // nw, nw * 64))
+    for name, gx, gy, threads in grids:
         waves = gx * gy * threads // 64
         empty = [(lambda: _lib.check(lib.exl3_diag_empty_launch(gx, gy, threads, stream()),
                                      "exl3_diag_empty_launch"))] * 64
