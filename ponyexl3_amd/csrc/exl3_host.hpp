@@ -116,14 +116,17 @@ int launch_had_post(const void* y, int y_is_fp32, int n_sum, size_t sum_stride, 
                     const uint16_t* svh, const uint16_t* bias, uint16_t* out, hipStream_t stream);
 
 // Tile schedule of the prefill GEMM: block tiles of (32*mi) rows x 256 columns are
-// dealt to the CUs in rounds; the `split_tiles` tiles of a partly filled last
-// round are cut into `split` reduction ranges of `ksteps_per_split` 64-deep steps
-// whose fp32 partial tiles a second kernel adds up.
+// dealt to the CUs in rounds; the `split_tiles` tiles of a partly filled last round
+// are cut along the reduction into `split_runs` runs of `split_per` 64-deep steps,
+// one workgroup each, whose fp32 partial tiles a second kernel adds up: either
+// `split_runs_per_tile` runs per tile, or (0) the tiles' steps end to end in equally
+// long runs that may cross from one tile into the next (`split_pitch`: positions from
+// one tile's first step to the next tile's).
 struct GemmPlan {
     int mi;  // 16-row accumulator tiles per wave: 8, 4 or 2 (256-, 128- or 64-row blocks)
     int n_row_blocks, n_col_blocks;
     int full_tiles, split_tiles;
-    int split, ksteps_per_split;
+    int split_runs, split_per, split_pitch, split_runs_per_tile;
 };
 GemmPlan plan_gemm(int rows, int in_tiles, int tn_count, bool allow_split);
 size_t gemm_workspace_bytes(int rows, int in_tiles, int tn_count);

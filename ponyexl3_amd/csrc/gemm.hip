@@ -27,9 +27,11 @@
 // ends up with 4 consecutive output columns of one row.
 //
 // Tail handling: tiles are dealt to CUs in rounds. The tiles of a last, partly
-// filled round are split along the reduction dimension into `split` ranges so
-// that the round costs 1/split of a tile time; those workgroups write fp32
-// partial tiles to a workspace and a small second kernel adds them in a fixed
+// filled round are not given a CU each: their 64-deep steps, laid end to end
+// (tile after tile), are cut into equal runs, one per CU, so that the round
+// costs rem/CUs of a tile time. A run that crosses a tile border works on two
+// tiles one after the other. Every piece writes an fp32 partial tile to a
+// workspace and a small second kernel adds the pieces of each tile in run
 // order and rounds once to fp16.
 //
 // Replaces the rows > 16 ladder of EXL3Linear.__call__
@@ -46,10 +48,28 @@ constexpr int kGemmStageB = kGemmBN * 64;
 
 __device__ __forceinline__ int lds_chunk_swizzle(int row) { return ((row >> 1) & 3) << 1; }
 
-// Work unit `unit` of the launch -> tile and reduction range.
+// One piece of work: a whole tile (partial_slot < 0, direct fp16 output) or a range
+// of a split tile's steps whose fp32 partial tile goes to slot `partial_slot`.
 struct GemmWork {
-    int tile, k_begin, k_end, partial_unit;  // partial_unit < 0: direct fp16 output
+    int tile, k_begin, k_end, partial_slot;
 };
+
+// The split region: every tile's `ksteps` steps sit at the start of a stretch of
+// `pitch` >= ksteps positions, the stretches end to end, cut into runs of `per`
+// positions (per <= pitch, so a run touches at most two tiles; the planner never
+// makes a run that starts in the unused end of a stretch). Two shapes are used:
+// pitch = ksteps, runs of any length that cross tile borders (as many runs as CUs,
+// all equally long), and pitch = s * per, s runs per tile that never cross.
+// Piece `si` (0 or 1) of run v covers tile j = first tile of the run + si; its
+// partial tile is slot v + j, which numbers the pieces in run order (slots < runs +
+// tiles). The pieces of tile j are those of runs first_run(j) .. last_run(j).
+// (tiles * pitch < 2^31: the planner does not split otherwise)
+__host__ __device__ __forceinline__ int split_first_run(int j, int pitch, int per) {
+    return (j * pitch) / per;
+}
+__host__ __device__ __forceinline__ int split_last_run(int j, int pitch, int ksteps, int per) {
+    return (j * pitch + ksteps - 1) / per;
+}
 
 // Workgroups are handed to the eight XCDs round-robin by index, and each XCD has
 // its own L2. Whole tiles are numbered column block first (tile = g * n_row_blocks
@@ -67,58 +87,131 @@ __device__ __forceinline__ int xcd_tile_order(int b, int full_tiles, int n_row_b
     return g * n_row_blocks + q % n_row_blocks;
 }
 
-__device__ __forceinline__ GemmWork gemm_work(int unit, int full_tiles, int split,
-                                              int ksteps_per_split, int ksteps,
-                                              int n_row_blocks, int split_units) {
+// Split geometry as the kernel gets it.
+struct GemmSplit {
+    int per, pitch, runs_per_tile;  // runs_per_tile > 0: runs never cross tiles
+    int positions;                  // tiles * pitch
+};
+
+// Number of pieces of workgroup `unit` and piece `si` of it.
+__device__ __forceinline__ int gemm_pieces(int unit, int full_tiles, const GemmSplit& sp) {
+    if (unit < full_tiles) return 1;
+    const int p0 = (unit - full_tiles) * sp.per;
+    const int p1 = min(p0 + sp.per, sp.positions);
+    return p1 - 1 >= (p0 / sp.pitch + 1) * sp.pitch ? 2 : 1;
+}
+
+__device__ __forceinline__ GemmWork gemm_work(int unit, int si, int full_tiles, int ksteps,
+                                              const GemmSplit& sp, int n_row_blocks,
+                                              int split_units) {
     GemmWork w;
     if (unit < full_tiles) {
         w.tile = xcd_tile_order(unit, full_tiles, n_row_blocks);
         w.k_begin = 0;
         w.k_end = ksteps;
-        w.partial_unit = -1;
+        w.partial_slot = -1;
     } else {
-        // Split tiles: the units that share trellis data are the row blocks of one
-        // (column block, reduction range) pair. Those pairs are numbered gv = column
-        // block * split + range, units v = gv * n_row_blocks + row block, and v is
-        // dealt to the XCDs like the whole tiles above.
-        int r = unit - full_tiles;  // canonical index: (tile - full_tiles) * split + range
-        if (full_tiles % n_row_blocks == 0) {
-            const int v = xcd_tile_order(r, split_units, n_row_blocks);
-            const int gv = v / n_row_blocks, rb = v % n_row_blocks;
-            r = ((gv / split) * n_row_blocks + rb) * split + gv % split;
+        int v = unit - full_tiles;
+        if (sp.runs_per_tile > 0 && full_tiles % n_row_blocks == 0) {
+            // The runs that share trellis data are the row blocks of one (column block,
+            // range) pair. Those pairs are numbered gv = column block * runs_per_tile +
+            // range, workgroups u = gv * n_row_blocks + row block, and u is dealt to the
+            // XCDs like the whole tiles above.
+            const int s = sp.runs_per_tile;
+            const int u = xcd_tile_order(v, split_units, n_row_blocks);
+            const int gv = u / n_row_blocks, rb = u % n_row_blocks;
+            v = ((gv / s) * n_row_blocks + rb) * s + gv % s;
         }
-        w.tile = full_tiles + r / split;
-        const int sp = r % split;
-        w.k_begin = sp * ksteps_per_split;
-        w.k_end = min(ksteps, w.k_begin + ksteps_per_split);
-        w.partial_unit = split > 1 ? r : -1;
+        const int p0 = v * sp.per;
+        const int p1 = min(p0 + sp.per, sp.positions);
+        const int j = p0 / sp.pitch + si;
+        const int t0 = j * sp.pitch;
+        w.tile = full_tiles + j;
+        w.k_begin = si ? 0 : p0 - t0;
+        w.k_end = min(p1 - t0, ksteps);
+        w.partial_slot = v + j;
     }
     return w;
 }
 
-template <int K, int CB, int MI>
-__global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
-    const uint32_t* __restrict__ trellis, const half_t* __restrict__ xh, half_t* __restrict__ y,
-    float* __restrict__ partial, int rows_arg, size_t ldx, size_t ldy, int in_tiles, int out_tiles,
-    int tn_offset_arg, int tn_count_arg, int n_row_blocks, int full_tiles, int split,
-    int ksteps_per_split, const int4* __restrict__ group_tab, int group_tiles, int n_groups,
-    const int* __restrict__ block_sub, size_t sub_stride, const half_t* __restrict__ post_svh,
-    const half_t* __restrict__ post_bias, half_t* __restrict__ post_out, size_t ldo) {
+// The kernel's arguments, as one block at the start of its argument segment.
+struct GemmArgs {
+    const uint32_t* trellis;
+    const half_t* xh;
+    half_t* y;
+    float* partial;
+    int rows;
+    size_t ldx, ldy;
+    int in_tiles, out_tiles, tn_offset, tn_count, n_row_blocks, full_tiles;
+    GemmSplit split;
+    const int4* group_tab;
+    int group_tiles, n_groups;
+    const int* block_sub;
+    size_t sub_stride;
+    const half_t* post_svh;
+    const half_t* post_bias;
+    half_t* post_out;
+    size_t ldo;
+};
+
+// TWO: the launch has runs that cross tile borders, i.e. workgroups with two pieces.
+template <int K, int CB, int MI, bool TWO>
+__global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(GemmArgs by_value) {
     extern __shared__ __attribute__((aligned(16))) half_t smem[];
     constexpr int BM = 32 * MI;
     constexpr int STAGE_A = BM * 64, STAGE_B = kGemmStageB;
     half_t* a_s = smem;
     half_t* b_s = smem + 2 * STAGE_A;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 2, wn = wave & 3;  // wave tile origin: rows wm*16*MI, columns wn*64
-    // Plain mode: work unit -> (column block g, row block) of one matrix, maybe one
-    // of several reduction ranges. Grouped mode (group_tab != NULL): the rows are
+    // Plain mode: workgroup -> (column block g, row block) of one matrix, whole, or
+    // one or two pieces of split tiles. Grouped mode (group_tab != NULL): the rows are
     // sorted into groups (experts) that each multiply their own `group_tiles` tile
     // columns; group_tab[b] = {group, first row, end row} of row block b (first ==
     // end marks an unused entry), blockIdx.x = b * n_col_blocks + g, whole reduction.
+    //
+    // A workgroup with two pieces reads its arguments again for the second one, from
+    // the argument segment through a pointer the compiler cannot see through: kept in
+    // registers across the first piece's main loop they would cost more scalar
+    // registers than there are, and the spills would land in the loop.
+    const GemmArgs __attribute__((address_space(4)))* args =
+        (const GemmArgs __attribute__((address_space(4)))*)__builtin_amdgcn_kernarg_segment_ptr();
+    (void)by_value;
+    int n_pieces = 1;
+    if constexpr (TWO) {
+        const GemmArgs __attribute__((address_space(4)))* a0 = args;
+        asm volatile("" : "+s"(a0));
+        const GemmSplit split = {a0->split.per, a0->split.pitch, a0->split.runs_per_tile,
+                                 a0->split.positions};
+        n_pieces = a0->group_tab ? 1 : gemm_pieces(blockIdx.x, a0->full_tiles, split);
+    }
+    for (int piece = 0; piece < n_pieces; piece++) {
+    const GemmArgs __attribute__((address_space(4)))* ap = args;
+    if constexpr (TWO) asm volatile("" : "+s"(ap));
+    const uint32_t* __restrict__ trellis = ap->trellis;
+    const half_t* __restrict__ xh = ap->xh;
+    half_t* __restrict__ y = ap->y;
+    float* __restrict__ partial = ap->partial;
+    const int rows_arg = ap->rows;
+    const size_t ldx = ap->ldx, ldy = ap->ldy;
+    const int in_tiles = ap->in_tiles, out_tiles = ap->out_tiles;
+    const int tn_offset_arg = ap->tn_offset, tn_count_arg = ap->tn_count;
+    const int n_row_blocks = ap->n_row_blocks, full_tiles = ap->full_tiles;
+    const int4* __restrict__ group_tab = ap->group_tab;
+    const int group_tiles = ap->group_tiles, n_groups = ap->n_groups;
+    const int* __restrict__ block_sub = ap->block_sub;
+    const size_t sub_stride = ap->sub_stride;
+    const half_t* __restrict__ post_svh = ap->post_svh;
+    const half_t* __restrict__ post_bias = ap->post_bias;
+    half_t* __restrict__ post_out = ap->post_out;
+    const size_t ldo = ap->ldo;
+    // (the lane's indices, too, are derived anew for every piece)
+    int tid = threadIdx.x;
+    if constexpr (TWO) asm volatile("" : "+v"(tid));
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 2, wn = wave & 3;  // wave tile origin: rows wm*16*MI, columns wn*64
     GemmWork work;
     int g, m0, rows, tn_offset, tn_count;
+    const half_t* xh_t = xh;
     if (group_tab) {
         const int n_col_blocks = (group_tiles + 15) >> 4;
         int4 t = group_tab[blockIdx.x / n_col_blocks];
@@ -129,15 +222,17 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
         work.tile = 0;
         work.k_begin = 0;
         work.k_end = in_tiles / 4;
-        work.partial_unit = -1;
+        work.partial_slot = -1;
         g = blockIdx.x % n_col_blocks;
         m0 = t.y;
         rows = t.z;
         tn_offset = tn_offset_arg + t.x * group_tiles;
         tn_count = group_tiles;
     } else {
-        work = gemm_work(blockIdx.x, full_tiles, split, ksteps_per_split, in_tiles / 4,
-                         n_row_blocks, (int)gridDim.x - full_tiles);
+        const GemmSplit split = {ap->split.per, ap->split.pitch, ap->split.runs_per_tile,
+                                 ap->split.positions};
+        work = gemm_work(blockIdx.x, piece, full_tiles, in_tiles / 4, split, n_row_blocks,
+                         (int)gridDim.x - full_tiles);
         g = work.tile / n_row_blocks;  // 256-column block inside the slice
         m0 = (work.tile % n_row_blocks) * BM;
         rows = rows_arg;
@@ -145,7 +240,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
         tn_count = tn_count_arg;
         // sibling-fused layers: every 256-column block multiplies the activations that
         // were rotated with its own member's suh, xh[row][block_sub[g]][:]
-        if (block_sub) xh += (size_t)block_sub[g] * sub_stride;
+        if (block_sub) xh_t += (size_t)block_sub[g] * sub_stride;
     }
     const int k_begin = work.k_begin, k_last = work.k_end - 1;
     const int nsteps = work.k_end - work.k_begin;
@@ -166,7 +261,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
         b_w[cs] = n * 64 + ((2 * tr) ^ lds_chunk_swizzle(n)) * 8;
     }
     // A tile: wave w copies rows w*4*MI .. +4*MI-1 with MI/2 direct loads of 8 rows each
-    const char* abase = reinterpret_cast<const char*>(xh + (size_t)m0 * ldx);
+    const char* abase = reinterpret_cast<const char*>(xh_t + (size_t)m0 * ldx);
     uint32_t a_off[MI / 2];
     {
         const int rl = lane >> 3;
@@ -329,7 +424,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
 
     // acc[i][j] is D^T: lane holds columns 4*(lane/16)+0..3 of row lane%16
     const int col0 = g * kGemmBN + wn * 64 + (lane >> 4) * 4;
-    if (post_out && work.partial_unit < 0) {
+    if (post_out && work.partial_slot < 0) {
         // Output transform of a whole tile inside the kernel (ponyexl3/ref/forward.py:41-45):
         // y16 = fp16(acc) goes to LDS, then Z = Y16 x H128 per 128-column block runs on the
         // matrix pipe as well - 128 more MFMAs per wave next to the 64 of every k-step, instead
@@ -414,10 +509,10 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
                 }
             }
         });
-        return;
+        return;  // a whole tile is a workgroup's only piece
     }
-    if (g * kGemmBN + wn * 64 >= tn_count * 16) return;  // upper half of a half-width last block
-    if (work.partial_unit < 0) {
+    if (g * kGemmBN + wn * 64 >= tn_count * 16) continue;  // upper half of a half-width last block
+    if (work.partial_slot < 0) {
 #pragma unroll
         for (int ii = 0; ii < MI; ii++) {
             const int r = m0 + wm * (16 * MI) + ii * 16 + fr;
@@ -434,7 +529,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
             }
         }
     } else {
-        float* pt = partial + (size_t)work.partial_unit * (BM * kGemmBN);
+        float* pt = partial + (size_t)work.partial_slot * (BM * kGemmBN);
 #pragma unroll
         for (int ii = 0; ii < MI; ii++) {
             const int rl = wm * (16 * MI) + ii * 16 + fr;
@@ -446,24 +541,28 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
             }
         }
     }
+    }  // pieces: every wave has passed the closing barrier of the last step, so the
+       // next piece's prologue may refill the LDS stages
 }
 
-// Sums the `split` fp32 partial tiles of every split tile in index order and
-// rounds once to fp16. grid = (split tiles, BM/8): a workgroup of 256 threads
-// finishes 8 rows x 256 columns, one float4 per thread and range.
+// Sums the fp32 partial tiles of every split tile in run order and rounds once to
+// fp16. grid = (split tiles, BM/8): a workgroup of 256 threads finishes 8 rows x
+// 256 columns, one float4 per thread and piece.
 template <int MI>
 __global__ __launch_bounds__(256) void gemm_fixup_kernel(const float* __restrict__ partial,
                                                          half_t* __restrict__ y, int rows,
                                                          size_t ldy, int tn_count,
                                                          int n_row_blocks, int full_tiles,
-                                                         int split) {
+                                                         int ksteps, int pitch, int per) {
     constexpr int BM = 32 * MI;
-    const int tile = full_tiles + blockIdx.x;
+    const int j = blockIdx.x;
+    const int tile = full_tiles + j;
     const int g = tile / n_row_blocks;
     const int m0 = (tile % n_row_blocks) * BM;
     const int c4 = (threadIdx.x & 63) * 4;
     if (g * kGemmBN + c4 >= tn_count * 16) return;
-    const float* p0 = partial + (size_t)blockIdx.x * split * (BM * kGemmBN);
+    const int v0 = split_first_run(j, pitch, per), v1 = split_last_run(j, pitch, ksteps, per);
+    const float* p0 = partial + (size_t)(v0 + j) * (BM * kGemmBN);
 #pragma unroll
     for (int it = 0; it < 2; it++) {
         const int rl = blockIdx.y * 8 + it * 4 + (threadIdx.x >> 6);
@@ -471,8 +570,8 @@ __global__ __launch_bounds__(256) void gemm_fixup_kernel(const float* __restrict
         const float* p = p0 + rl * kGemmBN + c4;
         float4_t s = *reinterpret_cast<const float4_t*>(p);
 #pragma unroll 4
-        for (int sp = 1; sp < split; sp++)
-            s = s + *reinterpret_cast<const float4_t*>(p + (size_t)sp * (BM * kGemmBN));
+        for (int v = 1; v <= v1 - v0; v++)
+            s = s + *reinterpret_cast<const float4_t*>(p + (size_t)v * (BM * kGemmBN));
         half4_t o;
         o.x = (half_t)s.x;
         o.y = (half_t)s.y;
@@ -490,18 +589,21 @@ __global__ __launch_bounds__(256) void gemm_fixup_kernel(const float* __restrict
 template <int MI>
 __global__ __launch_bounds__(256) void gemm_fixup_post_kernel(
     const float* __restrict__ partial, int rows, int tn_count, int n_row_blocks, int full_tiles,
-    int split, const half_t* __restrict__ svh, const half_t* __restrict__ bias,
+    int ksteps, int pitch, int per, const half_t* __restrict__ svh,
+    const half_t* __restrict__ bias,
     half_t* __restrict__ out, size_t ldo) {
     constexpr int BM = 32 * MI;
     constexpr float kScale = 0.088388347648318440550f;  // 1/sqrt(128)
-    const int tile = full_tiles + blockIdx.x;
+    const int tj = blockIdx.x;
+    const int tile = full_tiles + tj;
     const int g = tile / n_row_blocks;
     const int m0 = (tile % n_row_blocks) * BM;
     const int lane = threadIdx.x & 63;
     const int c4 = lane * 4;
     const int col = g * kGemmBN + c4;
     const bool col_ok = col < tn_count * 16;  // false in the upper half of a half-width last block
-    const float* p0 = partial + (size_t)blockIdx.x * split * (BM * kGemmBN);
+    const int v0 = split_first_run(tj, pitch, per), v1 = split_last_run(tj, pitch, ksteps, per);
+    const float* p0 = partial + (size_t)(v0 + tj) * (BM * kGemmBN);
 #pragma unroll
     for (int it = 0; it < 2; it++) {
         const int rl = blockIdx.y * 8 + it * 4 + (threadIdx.x >> 6);
@@ -510,8 +612,8 @@ __global__ __launch_bounds__(256) void gemm_fixup_post_kernel(
         if (col_ok) {
             const float* p = p0 + rl * kGemmBN + c4;
             s = *reinterpret_cast<const float4_t*>(p);
-            for (int sp = 1; sp < split; sp++)
-                s = s + *reinterpret_cast<const float4_t*>(p + (size_t)sp * (BM * kGemmBN));
+            for (int v = 1; v <= v1 - v0; v++)
+                s = s + *reinterpret_cast<const float4_t*>(p + (size_t)v * (BM * kGemmBN));
         }
         float v[4] = {(float)(half_t)s.x, (float)(half_t)s.y, (float)(half_t)s.z,
                       (float)(half_t)s.w};
@@ -579,37 +681,70 @@ GemmPlan plan_gemm(int rows, int in_tiles, int tn_count, bool allow_split) {
     const long long tiles = (long long)p.n_row_blocks * p.n_col_blocks;
     const int ksteps = in_tiles / 4;
     const int slots = gemm_slots();
-    p.full_tiles = (int)(tiles / slots * slots);
-    p.split = 1;
-    p.ksteps_per_split = ksteps;
-    const int rem = (int)(tiles - p.full_tiles);
-    if (allow_split && rem > 0) {
-        // Cost of the last round in tile times: its workgroups run in
-        // ceil(rem*s/slots) waves of 1/s tile each, and every range also writes (and
-        // the fix-up reads) one fp32 tile, about the time of 8 steps.
+    p.full_tiles = (int)tiles;
+    p.split_tiles = p.split_runs = 0;
+    p.split_per = ksteps;
+    p.split_pitch = ksteps;
+    p.split_runs_per_tile = 0;
+    const int rem = (int)(tiles % slots);
+    if (allow_split && rem > 0 && (long long)rem * ksteps * 2 < 0x7fffffffLL) {
+        // Cost of the last round in tile times; 1 if its tiles stay whole. Every piece
+        // also writes (and the fix-up reads) one fp32 tile and has a pipeline of its own
+        // to fill: about the time of 8 steps.
         const int max_split = env_int("EXL3_GEMM_MAX_SPLIT", 16, 1, 64);
-        const double partial_cost = 8.0 / ksteps;
-        double best = 1.0;
+        const double piece_cost = 8.0;
+        double best = 0.95;
+        // (a) s runs per tile, none crossing a border: ceil(rem*s/slots) rounds of them
         for (int s = 2; s <= max_split && ksteps / s >= 4; s++) {
             const int kps = (ksteps + s - 1) / s;
             if ((ksteps + kps - 1) / kps != s) continue;  // some range would be empty
             const double cost =
-                (double)(((long long)rem * s + slots - 1) / slots) * (1.0 / s + partial_cost);
+                (double)(((long long)rem * s + slots - 1) / slots) * (kps + piece_cost) / ksteps;
             if (cost < best - 1e-9) {
                 best = cost;
-                p.split = s;
-                p.ksteps_per_split = kps;
+                p.split_per = kps;
+                p.split_pitch = s * kps;
+                p.split_runs_per_tile = s;
+                p.split_runs = rem * s;
             }
         }
+        // (b) one run per CU over the steps end to end: the runs that cross a border
+        // work on two pieces
+        if (max_split > 1) {
+            const long long steps = (long long)rem * ksteps;
+            long long per = (steps + slots - 1) / slots;
+            const long long floor_per = (ksteps + max_split - 1) / max_split;
+            if (per < floor_per) per = floor_per;
+            if (per < 4) per = 4;
+            if (per < ksteps) {
+                const double cost = ((double)per + piece_cost * (ksteps % per ? 2 : 1)) / ksteps;
+                if (cost < best - 1e-9) {
+                    best = cost;
+                    p.split_per = (int)per;
+                    p.split_pitch = ksteps;
+                    p.split_runs_per_tile = 0;
+                    p.split_runs = (int)((steps + per - 1) / per);
+                }
+            }
+        }
+        if (best < 0.95) {
+            p.full_tiles = (int)(tiles - rem);
+            p.split_tiles = rem;
+        } else {
+            p.split_runs = 0;
+        }
     }
-    if (p.split == 1) p.full_tiles = (int)tiles;  // nothing to fix up
-    p.split_tiles = (int)(tiles - p.full_tiles);
     return p;
+}
+
+// fp32 partial tiles of the split region: slot = run + tile < runs + tiles
+static size_t gemm_partial_slots(const GemmPlan& p) {
+    return p.split_tiles ? (size_t)p.split_runs + p.split_tiles : 0;
 }
 
 size_t gemm_workspace_bytes(int rows, int in_tiles, int tn_count) {
     const GemmPlan p = plan_gemm(rows, in_tiles, tn_count, true);
-    return (size_t)p.split_tiles * p.split * (32 * p.mi) * kGemmBN * sizeof(float);
+    return gemm_partial_slots(p) * (32 * p.mi) * kGemmBN * sizeof(float);
 }
 
 template <int K, int CB, int MI>
@@ -622,17 +757,37 @@ static int launch_gemm_mi(const GemmPlan& p, const uint16_t* xh, int rows, size_
     constexpr size_t lds_stages = (2 * (size_t)(32 * MI) * 64 + 2 * (size_t)kGemmStageB) * sizeof(half_t);
     constexpr size_t lds_tile = (size_t)(32 * MI) * (kGemmBN + 8) * sizeof(half_t);
     constexpr size_t lds = lds_stages > lds_tile ? lds_stages : lds_tile;
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_kernel<K, CB, MI>),
+    const bool two = p.split_tiles > 0 && p.split_runs_per_tile == 0;
+    auto kernel = two ? gemm_kernel<K, CB, MI, true> : gemm_kernel<K, CB, MI, false>;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
         return EXL3_E_LAUNCH;
-    const unsigned units = (unsigned)(p.full_tiles + p.split_tiles * p.split);
-    gemm_kernel<K, CB, MI><<<dim3(units), dim3(kGemmThreads), lds, stream>>>(
-        reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<const half_t*>(xh),
-        reinterpret_cast<half_t*>(y_out), partial, rows, ldx, ldy, in_tiles, out_tiles, tn_offset,
-        tn_count, p.n_row_blocks, p.full_tiles, p.split, p.ksteps_per_split, nullptr, 0, 0,
-        block_sub, sub_stride, post ? reinterpret_cast<const half_t*>(post->svh) : nullptr,
-        post ? reinterpret_cast<const half_t*>(post->bias) : nullptr,
-        post ? reinterpret_cast<half_t*>(post->out) : nullptr, post ? post->ldo : 0);
+    const unsigned units = (unsigned)(p.full_tiles + p.split_runs);
+    GemmArgs a{};
+    a.trellis = reinterpret_cast<const uint32_t*>(trellis);
+    a.xh = reinterpret_cast<const half_t*>(xh);
+    a.y = reinterpret_cast<half_t*>(y_out);
+    a.partial = partial;
+    a.rows = rows;
+    a.ldx = ldx;
+    a.ldy = ldy;
+    a.in_tiles = in_tiles;
+    a.out_tiles = out_tiles;
+    a.tn_offset = tn_offset;
+    a.tn_count = tn_count;
+    a.n_row_blocks = p.n_row_blocks;
+    a.full_tiles = p.full_tiles;
+    a.split = GemmSplit{p.split_per, p.split_pitch, p.split_runs_per_tile,
+                        p.split_tiles * p.split_pitch};
+    a.block_sub = block_sub;
+    a.sub_stride = sub_stride;
+    if (post) {
+        a.post_svh = reinterpret_cast<const half_t*>(post->svh);
+        a.post_bias = reinterpret_cast<const half_t*>(post->bias);
+        a.post_out = reinterpret_cast<half_t*>(post->out);
+        a.ldo = post->ldo;
+    }
+    kernel<<<dim3(units), dim3(kGemmThreads), lds, stream>>>(a);
     if (int rc = launch_status()) return rc;
     if (post) {
         // whole tiles were transformed by the kernel itself; split tiles by the pass that
@@ -640,8 +795,8 @@ static int launch_gemm_mi(const GemmPlan& p, const uint16_t* xh, int rows, size_
         if (p.split_tiles > 0) {
             gemm_fixup_post_kernel<MI>
                 <<<dim3((unsigned)p.split_tiles, 4 * MI), dim3(256), 0, stream>>>(
-                    partial, rows, tn_count, p.n_row_blocks, p.full_tiles, p.split,
-                    reinterpret_cast<const half_t*>(post->svh),
+                    partial, rows, tn_count, p.n_row_blocks, p.full_tiles, in_tiles / 4,
+                    p.split_pitch, p.split_per, reinterpret_cast<const half_t*>(post->svh),
                     reinterpret_cast<const half_t*>(post->bias),
                     reinterpret_cast<half_t*>(post->out), post->ldo);
             return launch_status();
@@ -651,7 +806,7 @@ static int launch_gemm_mi(const GemmPlan& p, const uint16_t* xh, int rows, size_
     if (p.split_tiles > 0) {
         gemm_fixup_kernel<MI><<<dim3((unsigned)p.split_tiles, 4 * MI), dim3(256), 0, stream>>>(
             partial, reinterpret_cast<half_t*>(y_out), rows, ldy, tn_count, p.n_row_blocks,
-            p.full_tiles, p.split);
+            p.full_tiles, in_tiles / 4, p.split_pitch, p.split_per);
         return launch_status();
     }
     return EXL3_OK;
@@ -673,11 +828,10 @@ int launch_gemm(const uint16_t* xh, int rows, size_t ldx, const uint16_t* trelli
         return EXL3_E_BAD_SHAPE;
     if (ldx * 2 * 256 >= (1ull << 31)) return EXL3_E_BAD_SHAPE;  // 32-bit row offsets inside a block
     GemmPlan p = plan_gemm(rows, in_tiles, tn_count, workspace != nullptr);
-    const size_t need = (size_t)p.split_tiles * p.split * (32 * p.mi) * kGemmBN * sizeof(float);
+    const size_t need = gemm_partial_slots(p) * (32 * p.mi) * kGemmBN * sizeof(float);
     if (need > workspace_bytes || (reinterpret_cast<uintptr_t>(workspace) & 15))
         p = plan_gemm(rows, in_tiles, tn_count, false);
-    if ((long long)p.full_tiles + (long long)p.split_tiles * p.split > 0x7fffffffLL)
-        return EXL3_E_BAD_SHAPE;
+    if ((long long)p.full_tiles + (long long)p.split_runs > 0x7fffffffLL) return EXL3_E_BAD_SHAPE;
     float* partial = reinterpret_cast<float*>(workspace);
     // the output transform rides on the kernel's epilogue (whole tiles) and on the fix-up
     // (split tiles); it needs whole Hadamard blocks of the whole width
@@ -711,16 +865,28 @@ static int launch_gemm_grouped_mi(const uint16_t* xh, int n_rows, size_t ldx,
                                   const int32_t* group_tab, int n_row_blocks, uint16_t* y_out,
                                   size_t ldy, hipStream_t stream) {
     constexpr size_t lds = (2 * (size_t)(32 * MI) * 64 + 2 * (size_t)kGemmStageB) * sizeof(half_t);
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_kernel<K, CB, MI>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_kernel<K, CB, MI, false>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
         return EXL3_E_LAUNCH;
     const long long units = (long long)n_row_blocks * ((group_tiles + 15) / 16);
     if (units > 0x7fffffffLL) return EXL3_E_BAD_SHAPE;
-    gemm_kernel<K, CB, MI><<<dim3((unsigned)units), dim3(kGemmThreads), lds, stream>>>(
-        reinterpret_cast<const uint32_t*>(trellis), reinterpret_cast<const half_t*>(xh),
-        reinterpret_cast<half_t*>(y_out), nullptr, n_rows, ldx, ldy, in_tiles, out_tiles, tn_base,
-        group_tiles, 1, 0, 1, in_tiles / 4, reinterpret_cast<const int4*>(group_tab), group_tiles,
-        n_groups, nullptr, 0, nullptr, nullptr, nullptr, 0);
+    GemmArgs a{};
+    a.trellis = reinterpret_cast<const uint32_t*>(trellis);
+    a.xh = reinterpret_cast<const half_t*>(xh);
+    a.y = reinterpret_cast<half_t*>(y_out);
+    a.rows = n_rows;
+    a.ldx = ldx;
+    a.ldy = ldy;
+    a.in_tiles = in_tiles;
+    a.out_tiles = out_tiles;
+    a.tn_offset = tn_base;
+    a.tn_count = group_tiles;
+    a.n_row_blocks = 1;
+    a.split = GemmSplit{in_tiles / 4, in_tiles / 4, 0, 0};
+    a.group_tab = reinterpret_cast<const int4*>(group_tab);
+    a.group_tiles = group_tiles;
+    a.n_groups = n_groups;
+    gemm_kernel<K, CB, MI, false><<<dim3((unsigned)units), dim3(kGemmThreads), lds, stream>>>(a);
     return launch_status();
 }
 

@@ -144,10 +144,42 @@ def test_split_tiles_match_oracle_and_unsplit(cuda, oracle, rows):
     assert rel_l2(y0.cpu().numpy(), y1.cpu().numpy()) < 5e-4
 
 
+@pytest.mark.parametrize("rows,slots", [(300, 5), (100, 5), (40, 7)])
+def test_runs_that_cross_tile_borders(cuda, oracle, monkeypatch, rows, slots):
+    """With few workgroup slots the tiles of the last round are laid end to end and
+    cut into one run per slot, so that runs cross from one tile into the next (the
+    schedule of o_proj and down_proj at M = 2048, here forced on a small shape by the
+    slot count): whole tiles and two-piece workgroups in one launch, for the three
+    block heights; the plain GEMM and the whole layer (fix-up with the output transform)
+    against the oracle, twice for determinism."""
+    from ponyexl3_amd import ops
+
+    monkeypatch.setenv("EXL3_GEMM_SLOTS", str(slots))
+    rng = np.random.default_rng(4700 + rows)
+    tr_np = rng.integers(0, 65536, size=(512, 64, 64), dtype=np.uint16)  # 8192 -> 1024, K = 4
+    tr = ops.as_trellis_tensor(tr_np, cuda)
+    suh = np.where(rng.random(8192) > 0.5, -1, 1).astype(np.float16)
+    svh = np.where(rng.random(1024) > 0.5, -1, 1).astype(np.float16)
+    x_np = (rng.standard_normal((rows, 8192)) * 0.25).astype(np.float16)
+    x = _t(x_np, cuda)
+    print(f"gemm crossing runs rows={rows} slots={slots}", flush=True)
+    y1 = ops.inner_gemm(x, tr, 4, 0)
+    y2 = ops.inner_gemm(x, tr, 4, 0)
+    assert torch.equal(y1, y2)
+    w = oracle.decode_trellis(tr_np, 4, 0).astype(np.float64)
+    assert rel_l2(y1.cpu().numpy(), x_np.astype(np.float64) @ w) < 5e-4
+    z1 = ops.linear_forward(x, tr, 4, 0, _t(suh, cuda), _t(svh, cuda))
+    z2 = ops.linear_forward(x, tr, 4, 0, _t(suh, cuda), _t(svh, cuda))
+    assert torch.equal(z1, z2)
+    ref = oracle.linear_forward(tr_np, 4, 0, suh, svh, x_np)
+    assert rel_l2(z1.cpu().numpy(), ref) < 1e-3
+
+
 @pytest.mark.parametrize("n_in,n_out", [(17408, 5120), (5120, 34816)])
 def test_config3_split_shapes_against_decoded_weights(cuda, n_in, n_out):
-    """M = 2048 on down_proj (160 tiles, all split three ways) and gate+up
-    (1088 tiles: four full rounds and 64 tiles split four ways) against the
+    """M = 2048 on down_proj (160 tiles, their steps end to end in one run per CU, runs
+    crossing from one tile into the next) and gate+up (1088 tiles: four full rounds
+    and 64 tiles in four runs each) against the
     bit-exact decoded weights times xh in fp32."""
     from ponyexl3_amd import ops
 
