@@ -515,11 +515,15 @@ GemvPlan plan_linear_small(int rows, int in_tiles, int n_groups, int K) {
 // (column groups x partial rows per group x 128 columns x batch rows). Measured on
 // the 27B-class shapes at one row: 33 k (4096 -> 4096) 9.1 -> 6.8 us, q+k+v
 // 15.0 -> 13.2 us (205 k with half-block splits), 174 k (down) 20.7 -> 19.2 us, 348 k (gate+up) no gain; at 8 rows
-// (2.8 M) the step got 13 % slower.
+// (2.8 M) the step got 13 % slower. At two rows the partial-row reduction is the
+// more expensive one up to 8/3 of that limit (down 348 k: 20.6 -> 18.9 us, o_proj as
+// half blocks 327 k: 11.7 -> 11.2 us, gate+up 696 k: no loss; the step 83.0 -> 79.8 us);
+// at four rows neither limit gains (86.0 / 86.6 / 90.4 us at 300 k / 800 k / 1.6 M).
 bool linear_small_uses_atomics(int rows, int n_groups, GemvPlan plan) {
     static const int kMaxAtomics = env_int("EXL3_LINEAR_MAX_ATOMICS", 300000, 0, 1 << 30);
     if (plan.n_partials() > 255) return false;  // the count field has eight bits
-    return (long long)n_groups * plan.n_partials() * 128 * rows <= kMaxAtomics;
+    const long long limit = rows == 2 ? (long long)kMaxAtomics * 8 / 3 : kMaxAtomics;
+    return (long long)n_groups * plan.n_partials() * 128 * rows <= limit;
 }
 
 GemvPlan plan_linear_small_launch(int rows, int in_tiles, int n_groups, int K) {
