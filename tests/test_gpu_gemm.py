@@ -144,25 +144,26 @@ def test_split_tiles_match_oracle_and_unsplit(cuda, oracle, rows):
     assert rel_l2(y0.cpu().numpy(), y1.cpu().numpy()) < 5e-4
 
 
-@pytest.mark.parametrize("rows,slots", [(300, 5), (100, 5), (40, 7)])
-def test_runs_that_cross_tile_borders(cuda, oracle, monkeypatch, rows, slots):
+@pytest.mark.parametrize("rows,slots,n_out", [(300, 5, 1024), (100, 5, 1024), (40, 7, 1024), (300, 7, 1152)])
+def test_runs_that_cross_tile_borders(cuda, oracle, monkeypatch, rows, slots, n_out):
     """With few workgroup slots the tiles of the last round are laid end to end and
     cut into one run per slot, so that runs cross from one tile into the next (the
     schedule of o_proj and down_proj at M = 2048, here forced on a small shape by the
     slot count): whole tiles and two-piece workgroups in one launch, for the three
-    block heights; the plain GEMM and the whole layer (fix-up with the output transform)
-    against the oracle, twice for determinism."""
+    block heights, and with a half-width last column block among the split tiles
+    (1152 columns); the plain GEMM and the whole layer (fix-up with the output
+    transform) against the oracle, twice for determinism."""
     from ponyexl3_amd import ops
 
     monkeypatch.setenv("EXL3_GEMM_SLOTS", str(slots))
     rng = np.random.default_rng(4700 + rows)
-    tr_np = rng.integers(0, 65536, size=(512, 64, 64), dtype=np.uint16)  # 8192 -> 1024, K = 4
+    tr_np = rng.integers(0, 65536, size=(512, n_out // 16, 64), dtype=np.uint16)  # 8192 -> n_out, K = 4
     tr = ops.as_trellis_tensor(tr_np, cuda)
     suh = np.where(rng.random(8192) > 0.5, -1, 1).astype(np.float16)
-    svh = np.where(rng.random(1024) > 0.5, -1, 1).astype(np.float16)
+    svh = np.where(rng.random(n_out) > 0.5, -1, 1).astype(np.float16)
     x_np = (rng.standard_normal((rows, 8192)) * 0.25).astype(np.float16)
     x = _t(x_np, cuda)
-    print(f"gemm crossing runs rows={rows} slots={slots}", flush=True)
+    print(f"gemm crossing runs rows={rows} slots={slots} n_out={n_out}", flush=True)
     y1 = ops.inner_gemm(x, tr, 4, 0)
     y2 = ops.inner_gemm(x, tr, 4, 0)
     assert torch.equal(y1, y2)
