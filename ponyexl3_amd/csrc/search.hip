@@ -75,7 +75,6 @@ __global__ __launch_bounds__(256, 2) void quantize_tiles_kernel(const float* __r
     constexpr int KR = 16 - K, EDGES = 1 << KR, KK = 1 << K;
     constexpr int PER_LANE = EDGES / 256;             // states per lane
     constexpr int CH = PER_LANE < 8 ? PER_LANE : 8;   // states per LDS read
-    constexpr int NCH = PER_LANE / CH;
     // A cost row is stored in blocks of 256 states with PAD halfs between blocks:
     // the lanes of a wave write the states of 64 / 2^K different blocks at the same
     // offset, and unpadded those would all fall into the same LDS banks.

@@ -144,35 +144,38 @@ def test_split_tiles_match_oracle_and_unsplit(cuda, oracle, rows):
     assert rel_l2(y0.cpu().numpy(), y1.cpu().numpy()) < 5e-4
 
 
-@pytest.mark.parametrize("rows,slots,n_out", [(300, 5, 1024), (100, 5, 1024), (40, 7, 1024), (300, 7, 1152)])
-def test_runs_that_cross_tile_borders(cuda, oracle, monkeypatch, rows, slots, n_out):
+@pytest.mark.parametrize("rows,slots,n_out,k,cb", [
+    (300, 5, 1024, 4, 0), (100, 5, 1024, 4, 0), (40, 7, 1024, 4, 0), (300, 7, 1152, 4, 0),
+    (300, 5, 1024, 8, 2), (300, 5, 1024, 7, 1), (100, 5, 1024, 3, 0), (40, 7, 1024, 6, 1)])
+def test_runs_that_cross_tile_borders(cuda, oracle, monkeypatch, rows, slots, n_out, k, cb):
     """With few workgroup slots the tiles of the last round are laid end to end and
     cut into one run per slot, so that runs cross from one tile into the next (the
     schedule of o_proj and down_proj at M = 2048, here forced on a small shape by the
     slot count): whole tiles and two-piece workgroups in one launch, for the three
     block heights, and with a half-width last column block among the split tiles
-    (1152 columns); the plain GEMM and the whole layer (fix-up with the output
-    transform) against the oracle, twice for determinism."""
+    (1152 columns), and at other K / codebooks (K = 8 with MUL1 is the instantiation
+    with the most registers); the plain GEMM and the whole layer (fix-up with the
+    output transform) against the oracle, twice for determinism."""
     from ponyexl3_amd import ops
 
     monkeypatch.setenv("EXL3_GEMM_SLOTS", str(slots))
-    rng = np.random.default_rng(4700 + rows)
-    tr_np = rng.integers(0, 65536, size=(512, n_out // 16, 64), dtype=np.uint16)  # 8192 -> n_out, K = 4
+    rng = np.random.default_rng(4700 + rows + 10 * k + cb)
+    tr_np = rng.integers(0, 65536, size=(512, n_out // 16, 16 * k), dtype=np.uint16)  # 8192 -> n_out
     tr = ops.as_trellis_tensor(tr_np, cuda)
     suh = np.where(rng.random(8192) > 0.5, -1, 1).astype(np.float16)
     svh = np.where(rng.random(n_out) > 0.5, -1, 1).astype(np.float16)
     x_np = (rng.standard_normal((rows, 8192)) * 0.25).astype(np.float16)
     x = _t(x_np, cuda)
-    print(f"gemm crossing runs rows={rows} slots={slots} n_out={n_out}", flush=True)
-    y1 = ops.inner_gemm(x, tr, 4, 0)
-    y2 = ops.inner_gemm(x, tr, 4, 0)
+    print(f"gemm crossing runs rows={rows} slots={slots} n_out={n_out} k={k} cb={cb}", flush=True)
+    y1 = ops.inner_gemm(x, tr, k, cb)
+    y2 = ops.inner_gemm(x, tr, k, cb)
     assert torch.equal(y1, y2)
-    w = oracle.decode_trellis(tr_np, 4, 0).astype(np.float64)
+    w = oracle.decode_trellis(tr_np, k, cb).astype(np.float64)
     assert rel_l2(y1.cpu().numpy(), x_np.astype(np.float64) @ w) < 5e-4
-    z1 = ops.linear_forward(x, tr, 4, 0, _t(suh, cuda), _t(svh, cuda))
-    z2 = ops.linear_forward(x, tr, 4, 0, _t(suh, cuda), _t(svh, cuda))
+    z1 = ops.linear_forward(x, tr, k, cb, _t(suh, cuda), _t(svh, cuda))
+    z2 = ops.linear_forward(x, tr, k, cb, _t(suh, cuda), _t(svh, cuda))
     assert torch.equal(z1, z2)
-    ref = oracle.linear_forward(tr_np, 4, 0, suh, svh, x_np)
+    ref = oracle.linear_forward(tr_np, k, cb, suh, svh, x_np)
     assert rel_l2(z1.cpu().numpy(), ref) < 1e-3
 
 
