@@ -1,5 +1,7 @@
 """EXL3Linear / FusedEXL3Group against the oracle's layer forward
 (rel-L2 <= 1e-3, fp32 accumulation)."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -246,6 +248,8 @@ def test_bounded_wait_gives_up_visibly(cuda, monkeypatch):
     call is right again."""
     from ponyexl3_amd import make_exl3_layer, ops
 
+    if os.environ.get("EXL3_EXACT_WEIGHTS") == "1":
+        pytest.skip("the multi-launch chains this knob selects have no accumulator reduction")
     layer = make_exl3_layer(k=4, in_features=1024, out_features=384, seed=97)
     tr = ops.as_trellis_tensor(layer.trellis, cuda)
     suh, svh = torch.from_numpy(layer.suh).to(cuda), torch.from_numpy(layer.svh).to(cuda)
@@ -253,19 +257,23 @@ def test_bounded_wait_gives_up_visibly(cuda, monkeypatch):
     good = ops.linear_forward(xt, tr, 4, 0, suh, svh, fused=True)
     ops.check_counters(cuda)
     cnt = ops.sync_counters(cuda, 1)
-    # accumulator of (row 0, column 128 + 5): a count of 255 before anybody has added
-    cnt.view(torch.int64)[128 + 5] = -(1 << 56)
-    monkeypatch.setenv("EXL3_SPIN_LIMIT", "4")
-    print("linear bounded wait", flush=True)
-    bad = ops.linear_forward(xt, tr, 4, 0, suh, svh, fused=True)
-    torch.cuda.synchronize()
-    assert torch.isnan(bad[:, 128:256].float()).all()
-    assert torch.equal(bad[:, :128], good[:, :128]) and torch.equal(bad[:, 256:], good[:, 256:])
-    with pytest.raises(RuntimeError):
+    try:
+        # accumulator of (row 0, column 128 + 5): a count of 255 before anybody has added
+        cnt.view(torch.int64)[128 + 5] = -(1 << 56)
+        monkeypatch.setenv("EXL3_SPIN_LIMIT", "4")
+        print("linear bounded wait", flush=True)
+        bad = ops.linear_forward(xt, tr, 4, 0, suh, svh, fused=True)
+        torch.cuda.synchronize()
+        assert torch.isnan(bad[:, 128:256].float()).all()
+        assert torch.equal(bad[:, :128], good[:, :128]) and torch.equal(bad[:, 256:], good[:, 256:])
+        with pytest.raises(RuntimeError):
+            ops.check_counters(cuda)
+        monkeypatch.delenv("EXL3_SPIN_LIMIT")
+        assert torch.equal(ops.linear_forward(xt, tr, 4, 0, suh, svh, fused=True), good)
         ops.check_counters(cuda)
-    monkeypatch.delenv("EXL3_SPIN_LIMIT")
-    assert torch.equal(ops.linear_forward(xt, tr, 4, 0, suh, svh, fused=True), good)
-    ops.check_counters(cuda)
+    finally:
+        torch.cuda.synchronize()
+        cnt.zero_()  # whatever happened above, the shared array is clean for the next test
 
 
 def test_sibling_cache_under_inference_mode(cuda):

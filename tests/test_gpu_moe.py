@@ -1,4 +1,6 @@
 """Routed MoE expert chain against the oracle's unfused per-expert chain."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -248,6 +250,8 @@ def test_bounded_wait_gives_up_visibly(cuda, monkeypatch):
     slot's output is NaN, the other slots are untouched and the status word is set."""
     from ponyexl3_amd import EXL3SwitchGLU, ops
 
+    if os.environ.get("EXL3_EXACT_WEIGHTS") == "1":
+        pytest.skip("the multi-launch chains this knob selects have no accumulator reduction")
     E, D, H, kk, k = 4, 640, 256, 2, 4
     gate, up, down = _experts(E, D, H, k, False, 900)
     moe = EXL3SwitchGLU.from_layers(gate, up, down)
@@ -259,19 +263,23 @@ def test_bounded_wait_gives_up_visibly(cuda, monkeypatch):
     good = ops.moe_forward(*args, fused=True)
     ops.check_counters(cuda)
     cnt = ops.sync_counters(cuda, 1)
-    # accumulator of (slot 0, gate, column 5): a count of 255 that can never come out right
-    cnt.view(torch.int64)[5] = -(1 << 56)
-    monkeypatch.setenv("EXL3_SPIN_LIMIT", "4")
-    print("moe bounded wait", flush=True)
-    bad = ops.moe_forward(*args, fused=True)
-    torch.cuda.synchronize()
-    assert torch.isnan(bad[0, 0].float()).all()
-    assert torch.equal(bad[0, 1], good[0, 1])
-    with pytest.raises(RuntimeError):
+    try:
+        # accumulator of (slot 0, gate, column 5): a count of 255 that can never come out right
+        cnt.view(torch.int64)[5] = -(1 << 56)
+        monkeypatch.setenv("EXL3_SPIN_LIMIT", "4")
+        print("moe bounded wait", flush=True)
+        bad = ops.moe_forward(*args, fused=True)
+        torch.cuda.synchronize()
+        assert torch.isnan(bad[0, 0].float()).all()
+        assert torch.equal(bad[0, 1], good[0, 1])
+        with pytest.raises(RuntimeError):
+            ops.check_counters(cuda)
+        monkeypatch.delenv("EXL3_SPIN_LIMIT")
+        assert torch.equal(ops.moe_forward(*args, fused=True), good)  # check_counters zeroed the array
         ops.check_counters(cuda)
-    monkeypatch.delenv("EXL3_SPIN_LIMIT")
-    assert torch.equal(ops.moe_forward(*args, fused=True), good)  # check_counters zeroed the array
-    ops.check_counters(cuda)
+    finally:
+        torch.cuda.synchronize()
+        cnt.zero_()  # whatever happened above, the shared array is clean for the next test
 
 
 def test_config4_a3b_shapes(cuda, oracle):
