@@ -27,12 +27,14 @@
 // ends up with 4 consecutive output columns of one row.
 //
 // Tail handling: tiles are dealt to CUs in rounds. The tiles of a last, partly
-// filled round are not given a CU each: their 64-deep steps, laid end to end
-// (tile after tile), are cut into equal runs, one per CU, so that the round
-// costs rem/CUs of a tile time. A run that crosses a tile border works on two
-// tiles one after the other. Every piece writes an fp32 partial tile to a
-// workspace and a small second kernel adds the pieces of each tile in run
-// order and rounds once to fp16.
+// filled round are not given a CU each but cut along the reduction into runs of
+// 64-deep steps, one workgroup per run; the planner takes the cheaper of two
+// shapes: s runs per tile (in as many rounds as rem*s runs need), or the tiles'
+// steps laid end to end and cut into equal runs, one per CU, so that the round
+// costs rem/CUs of a tile time - a run that crosses a tile border then works on
+// two tiles one after the other (kernel instantiation TWO). Every piece writes an
+// fp32 partial tile to a workspace and a small second kernel adds the pieces of
+// each tile in run order and rounds once to fp16.
 //
 // Replaces the rows > 16 ladder of EXL3Linear.__call__
 // (ponyexl3/mlx/exl3_linear.py:137-161) and the decode-into-threadgroup-memory
