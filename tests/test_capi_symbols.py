@@ -116,6 +116,36 @@ def test_workspace_sizes(lib):
     assert lib.exl3_moe_workspace_bytes(1, 8, 2048, 500) == 0
 
 
+def test_gemm_split_plan_sizes(lib, monkeypatch):
+    """The prefill GEMM's split plan (host arithmetic only): the workspace it asks for
+    is whole fp32 partial tiles, at most one per run plus one per split tile, for any
+    shape and any number of workgroup slots; nothing is asked for when the tiles fill
+    whole rounds of the slots."""
+    def tiles_of(rows, tn):
+        mi = 2 if rows <= 64 else 4 if rows <= 128 else 8
+        bm = 32 * mi
+        return (rows + bm - 1) // bm * ((tn + 15) // 16), bm * 256 * 4
+
+    for slots in (1, 3, 7, 64, 256, 304):
+        monkeypatch.setenv("EXL3_GEMM_SLOTS", str(slots))
+        for rows in (17, 64, 100, 128, 300, 2048, 5000):
+            for in_tiles in (4, 8, 64, 320, 1088, 4096):
+                for tn in (8, 24, 64, 320, 2176):
+                    nbytes = int(lib.exl3_gemm_workspace_bytes(rows, in_tiles, tn))
+                    tiles, tile_bytes = tiles_of(rows, tn)
+                    rem = tiles % slots
+                    assert nbytes % tile_bytes == 0
+                    # runs <= max(slots, 16 * rem) (one per slot, or up to 16 per tile), + rem
+                    assert nbytes // tile_bytes <= max(slots, 16 * rem) + rem
+                    if rem == 0:
+                        assert nbytes == 0
+    monkeypatch.setenv("EXL3_GEMM_SLOTS", "256")
+    # config 3: o_proj / down_proj (160 tiles: one run per CU, 415 / 416 slots reserved),
+    # gate+up (64 tiles in four runs each)
+    assert int(lib.exl3_gemm_workspace_bytes(2048, 512, 320)) == (256 + 160) * 256 * 256 * 4
+    assert int(lib.exl3_gemm_workspace_bytes(2048, 320, 2176)) == (256 + 64) * 256 * 256 * 4
+
+
 def test_status_to_exception():
     from ponyexl3_amd import _lib
 
